@@ -1,4 +1,4 @@
-from . import llama  # noqa: F401  (registers the architecture, its adapters and variants)
+from . import llama, zodolorn  # noqa: F401  (register the architectures, their adapters and variants)
 from .registry import (
     Architecture,
     architecture_for_hf,

@@ -38,6 +38,8 @@ def register_architecture(arch: Architecture) -> None:
 
 
 def get_architecture(name: str) -> Architecture:
+    if name not in _architectures and str(name).lower() in _architectures:
+        name = str(name).lower()  # a config.json may write the name with capitals
     if name not in _architectures:
         raise KeyError(f"{name} is not registered; known architectures: {list_models()}")
     return _architectures[name]

@@ -34,6 +34,9 @@ class KVNeed:
     kv_heads: int
     head_dim: int
     window: int = 0  # 0: all keys; w > 0: the last w keys
+    # False: one tensor of rows [page][kv head][token][head_dim] and no value tensor (a mixer whose values are a part
+    # or a function of what it keeps as keys, like attention over a latent)
+    values: bool = True
 
 
 @dataclasses.dataclass(frozen=True)
@@ -60,10 +63,11 @@ class KVGroup:
         n, K, D = self.pool.n_pages, self.need.kv_heads, self.need.head_dim
         # zero-filled: the attention kernels multiply masked-out positions by zero
         self.keys = torch.zeros(len(self.entries), n, K, PAGE_TOKENS, D, dtype=dtype, device=device)
-        self.values = torch.zeros(len(self.entries), n, K, D, PAGE_TOKENS, dtype=dtype, device=device)
+        if self.need.values:
+            self.values = torch.zeros(len(self.entries), n, K, D, PAGE_TOKENS, dtype=dtype, device=device)
 
     def bytes_per_token(self, itemsize: int) -> int:
-        return 2 * len(self.entries) * self.need.kv_heads * self.need.head_dim * itemsize
+        return (2 if self.need.values else 1) * len(self.entries) * self.need.kv_heads * self.need.head_dim * itemsize
 
 
 class SequenceCache:
@@ -256,10 +260,10 @@ class SequenceCache:
 
     # ---- storage views -----------------------------------------------------
     def kv_of_entry(self, entry: int) -> Tuple[int, torch.Tensor, torch.Tensor]:
-        """(group index, keys [pages, K, 64, D], values [pages, K, D, 64]) of a schedule entry."""
+        """(group index, keys [pages, K, 64, D], values [pages, K, D, 64] or None) of a schedule entry."""
         g, i = self.group_of_entry[entry]
         group = self.groups[g]
-        return g, group.keys[i], group.values[i]
+        return g, group.keys[i], group.values[i] if group.values is not None else None
 
     def state_of_entry(self, entry: int) -> Dict[str, torch.Tensor]:
         return self.state.get(entry, {})

@@ -1,4 +1,5 @@
 from .base import ModelConfig
 from .llama import LLaMAConfig
+from .zodolorn import ZodolornConfig
 
-__all__ = ["ModelConfig", "LLaMAConfig"]
+__all__ = ["ModelConfig", "LLaMAConfig", "ZodolornConfig"]

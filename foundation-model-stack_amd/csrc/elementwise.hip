@@ -23,28 +23,28 @@ extern "C" const char* fmsamd_last_error() { return g_error; }
 extern "C" int fmsamd_abi_version() { return FMSAMD_ABI_VERSION; }
 
 // --------------------------------------------------------------------------
-// embedding: resid[t, :] = float(table[ids[t], :])
+// embedding: resid[t, :] = float(table[ids[t], :]) * scale
 // --------------------------------------------------------------------------
 template <typename TableT>
 __global__ void embed_kernel(const int* __restrict__ ids, const TableT* __restrict__ table, float* __restrict__ out,
-                             int width, int vocab) {
+                             int width, int vocab, float scale) {
   const int t = blockIdx.x;
   int id = ids[t];
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);  // the host has checked the range; never read outside
   const TableT* row = table + (size_t)id * width;
   float* o = out + (size_t)t * width;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = to_f32(row[i]);
+  for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = to_f32(row[i]) * scale;
 }
 
 extern "C" int fmsamd_embed(const int* ids, const void* table, int table_dtype, float* out, int n_tokens, int width,
-                            int vocab, hipStream_t stream) {
+                            int vocab, float scale, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   FMS_REQUIRE(n_tokens > 0 && width > 0 && vocab > 0, "embed: bad sizes T=%d width=%d vocab=%d", n_tokens, width, vocab);
   const int threads = width >= 1024 ? 256 : 64;
   if (table_dtype == FMS_F32)
-    embed_kernel<float><<<n_tokens, threads, 0, stream>>>(ids, (const float*)table, out, width, vocab);
+    embed_kernel<float><<<n_tokens, threads, 0, stream>>>(ids, (const float*)table, out, width, vocab, scale);
   else if (table_dtype == FMS_BF16)
-    embed_kernel<bf16><<<n_tokens, threads, 0, stream>>>(ids, (const bf16*)table, out, width, vocab);
+    embed_kernel<bf16><<<n_tokens, threads, 0, stream>>>(ids, (const bf16*)table, out, width, vocab, scale);
   else
     FMS_REQUIRE(false, "embed: unknown table dtype %d", table_dtype);
   FMS_LAUNCH_CHECK("embed");

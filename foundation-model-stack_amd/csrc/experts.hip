@@ -1,0 +1,295 @@
+// A feed-forward of many small experts of which every token uses a few.
+//
+//   route:    float32 router logits [T, E] -> the `top` largest per token (ties: the lower index) and the softmax over
+//             those `top` logits alone.
+//   group:    the T * top (token, choice) pairs sorted by expert, cut into tiles of 16 rows that belong to one expert
+//             each.  It runs on the device, in one block, so a step never waits for the host (and can be captured).
+//   gate_up:  for every tile, hidden = clamp-gated activation of (x Wg_e^T, x Wu_e^T)
+//   down:     for every tile, y[pair] = hidden Wd_e^T, float32, at the pair's own place (token * top + choice)
+//   combine:  out[t] = sum_j weight[t, j] y[t * top + j]  (+ sigmoid(shared_gate[t]) * shared[t]), summed in the order
+//             of j: a token's result does not depend on what else is in the batch.
+//
+// The products take their rows through tile_product.h: float32 FMA for the 32-bit path, MFMA 16x16x32 for bfloat16.
+// The grids are sized for the worst case (every expert with a ragged last tile); tiles that do not exist leave at once.
+#include "common.h"
+#include "fmsamd.h"
+#include "tile_product.h"
+
+#define ROUTE_MAX_EXPERTS 1024
+#define ROUTE_MAX_TOP 64
+
+// One wave per token.
+__global__ void __launch_bounds__(256)
+    route_kernel(const float* __restrict__ logits, long ld, int n_tokens, int n_experts, int top, int* __restrict__ ids,
+                 float* __restrict__ weights) {
+  extern __shared__ float lds[];  // 4 waves x (n_experts + top)
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= n_tokens) return;
+  float* z = lds + (size_t)wave * (n_experts + top);
+  float* chosen = z + n_experts;
+  for (int e = lane; e < n_experts; e += WAVE) z[e] = logits[(size_t)t * ld + e];
+  __builtin_amdgcn_wave_barrier();
+  for (int j = 0; j < top; ++j) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+    for (int e = lane; e < n_experts; e += WAVE) {
+      const float v = z[e];
+      if (v > best || (v == best && e < at)) best = v, at = e;
+    }
+    if (at == 0x7fffffff) at = lane < n_experts ? lane : 0;  // only NaNs or -inf left in this lane's share
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) {
+      const float ov = __shfl_xor(best, off, WAVE);
+      const int oa = __shfl_xor(at, off, WAVE);
+      if (ov > best || (ov == best && oa < at)) best = ov, at = oa;
+    }
+    if (lane == 0) {
+      ids[(size_t)t * top + j] = at;
+      chosen[j] = best;
+      z[at] = -INFINITY;
+    }
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
+  }
+  if (lane == 0) {
+    const float m = chosen[0];  // the largest comes first
+    float sum = 0.f;
+    for (int j = 0; j < top; ++j) sum += expf(chosen[j] - m);
+    for (int j = 0; j < top; ++j) weights[(size_t)t * top + j] = expf(chosen[j] - m) / sum;
+  }
+}
+
+extern "C" int fmsamd_moe_route(const float* logits, long ld, int n_tokens, int n_experts, int top, int* ids, float* weights,
+                                hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  FMS_REQUIRE(n_tokens > 0 && n_experts > 0 && n_experts <= ROUTE_MAX_EXPERTS && top > 0 && top <= n_experts && top <= ROUTE_MAX_TOP,
+              "moe_route: %d experts (at most %d), top %d (at most %d and the experts)", n_experts, ROUTE_MAX_EXPERTS, top, ROUTE_MAX_TOP);
+  FMS_REQUIRE(ld >= n_experts, "moe_route: rows of %ld for %d experts", ld, n_experts);
+  const size_t lds = 4 * (size_t)(n_experts + top) * sizeof(float);
+  route_kernel<<<ceil_div(n_tokens, 4), 256, lds, stream>>>(logits, ld, n_tokens, n_experts, top, ids, weights);
+  FMS_LAUNCH_CHECK("moe_route");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// group: order[0 .. n) = the pairs sorted by expert; tiles[i] = (expert, first row in order, rows), rows 0: no tile
+// --------------------------------------------------------------------------
+__global__ void __launch_bounds__(1024)
+    group_kernel(const int* __restrict__ ids, int n_pairs, int n_experts, int* __restrict__ order, int* __restrict__ tiles,
+                 int max_tiles) {
+  __shared__ int counts[ROUTE_MAX_EXPERTS];
+  __shared__ int cursor[ROUTE_MAX_EXPERTS];
+  for (int e = threadIdx.x; e < n_experts; e += blockDim.x) counts[e] = 0;
+  __syncthreads();
+  for (int a = threadIdx.x; a < n_pairs; a += blockDim.x) {
+    const int e = ids[a];
+    if (e >= 0 && e < n_experts) atomicAdd(&counts[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, nt = 0;
+    for (int e = 0; e < n_experts; ++e) {
+      cursor[e] = at;
+      const int c = counts[e];
+      for (int r = 0; r < c && nt < max_tiles; r += TILE_ROWS, ++nt) {
+        tiles[3 * nt] = e;
+        tiles[3 * nt + 1] = at + r;
+        tiles[3 * nt + 2] = c - r < TILE_ROWS ? c - r : TILE_ROWS;
+      }
+      at += c;
+    }
+    for (; nt < max_tiles; ++nt) tiles[3 * nt] = 0, tiles[3 * nt + 1] = 0, tiles[3 * nt + 2] = 0;
+  }
+  __syncthreads();
+  for (int a = threadIdx.x; a < n_pairs; a += blockDim.x) {
+    const int e = ids[a];
+    if (e >= 0 && e < n_experts) order[atomicAdd(&cursor[e], 1)] = a;
+  }
+}
+
+extern "C" int fmsamd_moe_max_tiles(int n_pairs, int n_experts) {
+  return (n_pairs + TILE_ROWS - 1) / TILE_ROWS + (n_experts < n_pairs ? n_experts : n_pairs);
+}
+
+extern "C" int fmsamd_moe_group(const int* ids, int n_pairs, int n_experts, int* order, int* tiles, int max_tiles,
+                                hipStream_t stream) {
+  if (n_pairs == 0) return 0;
+  FMS_REQUIRE(n_pairs > 0 && n_experts > 0 && n_experts <= ROUTE_MAX_EXPERTS, "moe_group: %d pairs, %d experts (at most %d)", n_pairs,
+              n_experts, ROUTE_MAX_EXPERTS);
+  FMS_REQUIRE(max_tiles >= fmsamd_moe_max_tiles(n_pairs, n_experts), "moe_group: room for %d tiles, %d may be needed", max_tiles,
+              fmsamd_moe_max_tiles(n_pairs, n_experts));
+  group_kernel<<<1, 1024, 0, stream>>>(ids, n_pairs, n_experts, order, tiles, max_tiles);
+  FMS_LAUNCH_CHECK("moe_group");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// the experts' products
+// --------------------------------------------------------------------------
+struct ExpertArgs {
+  const void* x;  // gate_up: [T, ldx] token rows; down: hidden [pairs, ldx] in sorted order
+  long ldx;
+  const void* w1;  // gate_up: gate weights [E, N, K]; down: down weights [E, N, K]
+  const void* w2;  // gate_up: up weights [E, N, K]
+  void* y;  // gate_up: hidden [pairs, N] in sorted order; down: float32 [pairs, N] by pair
+  const int* order;
+  const int* tiles;
+  int top, N, K;
+  float limit, alpha, shift;
+};
+
+__device__ __forceinline__ float clamp_gated(float g, float u, float limit, float alpha, float shift) {
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  return g / (1.f + expf(-alpha * g)) * (u + shift);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(TILE_THREADS) expert_gate_up_fma_kernel(ExpertArgs a) {
+  const int e = a.tiles[3 * blockIdx.x], start = a.tiles[3 * blockIdx.x + 1], rows = a.tiles[3 * blockIdx.x + 2];
+  if (rows == 0) return;
+  const int n0 = blockIdx.y * TILE_FMA_COLS;
+  const T* x = (const T*)a.x;
+  const T* wg = (const T*)a.w1 + (size_t)e * a.N * a.K;
+  const T* wu = (const T*)a.w2 + (size_t)e * a.N * a.K;
+  auto a_row = [&](int m) { return m < rows ? x + (size_t)(a.order[start + m] / a.top) * a.ldx : (const T*)nullptr; };
+  float g[4], u[4];
+  tile_product_fma<T>(a_row, [&](int n) { return n0 + n < a.N ? wg + (size_t)(n0 + n) * a.K : (const T*)nullptr; }, a.K, g);
+  tile_product_fma<T>(a_row, [&](int n) { return n0 + n < a.N ? wu + (size_t)(n0 + n) * a.K : (const T*)nullptr; }, a.K, u);
+  const int n = n0 + threadIdx.x % 64;
+  if (n >= a.N) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = (threadIdx.x / 64) * 4 + i;
+    if (m < rows) ((T*)a.y)[(size_t)(start + m) * a.N + n] = from_f32<T>(clamp_gated(g[i], u[i], a.limit, a.alpha, a.shift));
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(TILE_THREADS) expert_down_fma_kernel(ExpertArgs a) {
+  const int e = a.tiles[3 * blockIdx.x], start = a.tiles[3 * blockIdx.x + 1], rows = a.tiles[3 * blockIdx.x + 2];
+  if (rows == 0) return;
+  const int n0 = blockIdx.y * TILE_FMA_COLS;
+  const T* x = (const T*)a.x;
+  const T* w = (const T*)a.w1 + (size_t)e * a.N * a.K;
+  float acc[4];
+  tile_product_fma<T>([&](int m) { return m < rows ? x + (size_t)(start + m) * a.ldx : (const T*)nullptr; },
+                      [&](int n) { return n0 + n < a.N ? w + (size_t)(n0 + n) * a.K : (const T*)nullptr; }, a.K, acc);
+  const int n = n0 + threadIdx.x % 64;
+  if (n >= a.N) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = (threadIdx.x / 64) * 4 + i;
+    if (m < rows) ((float*)a.y)[(size_t)a.order[start + m] * a.N + n] = acc[i];
+  }
+}
+
+__global__ void __launch_bounds__(TILE_THREADS) expert_gate_up_mfma_kernel(ExpertArgs a) {
+  const int e = a.tiles[3 * blockIdx.x], start = a.tiles[3 * blockIdx.x + 1], rows = a.tiles[3 * blockIdx.x + 2];
+  if (rows == 0) return;
+  const int n0 = blockIdx.y * TILE_MFMA_COLS;
+  const bf16* x = (const bf16*)a.x;
+  const bf16* wg = (const bf16*)a.w1 + (size_t)e * a.N * a.K;
+  const bf16* wu = (const bf16*)a.w2 + (size_t)e * a.N * a.K;
+  auto a_row = [&](int m) { return m < rows ? x + (size_t)(a.order[start + m] / a.top) * a.ldx : (const bf16*)nullptr; };
+  f32x4 g[4], u[4];
+  tile_product_mfma(a_row, [&](int n) { return n0 + n < a.N ? wg + (size_t)(n0 + n) * a.K : (const bf16*)nullptr; }, a.K, g);
+  tile_product_mfma(a_row, [&](int n) { return n0 + n < a.N ? wu + (size_t)(n0 + n) * a.K : (const bf16*)nullptr; }, a.K, u);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = (lane >> 4) * 4 + i;
+    if (m >= rows) continue;
+#pragma unroll
+    for (int tl = 0; tl < 4; ++tl) {
+      const int n = n0 + wave * 64 + tl * 16 + (lane & 15);
+      if (n < a.N) ((bf16*)a.y)[(size_t)(start + m) * a.N + n] = (bf16)clamp_gated(g[tl][i], u[tl][i], a.limit, a.alpha, a.shift);
+    }
+  }
+}
+
+__global__ void __launch_bounds__(TILE_THREADS) expert_down_mfma_kernel(ExpertArgs a) {
+  const int e = a.tiles[3 * blockIdx.x], start = a.tiles[3 * blockIdx.x + 1], rows = a.tiles[3 * blockIdx.x + 2];
+  if (rows == 0) return;
+  const int n0 = blockIdx.y * TILE_MFMA_COLS;
+  const bf16* x = (const bf16*)a.x;
+  const bf16* w = (const bf16*)a.w1 + (size_t)e * a.N * a.K;
+  f32x4 acc[4];
+  tile_product_mfma([&](int m) { return m < rows ? x + (size_t)(start + m) * a.ldx : (const bf16*)nullptr; },
+                    [&](int n) { return n0 + n < a.N ? w + (size_t)(n0 + n) * a.K : (const bf16*)nullptr; }, a.K, acc);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = (lane >> 4) * 4 + i;
+    if (m >= rows) continue;
+    float* yrow = (float*)a.y + (size_t)a.order[start + m] * a.N;
+#pragma unroll
+    for (int tl = 0; tl < 4; ++tl) {
+      const int n = n0 + wave * 64 + tl * 16 + (lane & 15);
+      if (n < a.N) yrow[n] = acc[tl][i];
+    }
+  }
+}
+
+// stage 0: hidden = act(x Wg^T, x Wu^T) for the tiles' rows; stage 1: y = hidden Wd^T
+extern "C" int fmsamd_moe_experts(int stage, const void* x, long ldx, const void* w1, const void* w2, void* y, int dtype,
+                                  const int* order, const int* tiles, int max_tiles, int top, int N, int K, float limit,
+                                  float alpha, float shift, hipStream_t stream) {
+  if (max_tiles == 0) return 0;
+  FMS_REQUIRE(stage == 0 || stage == 1, "moe_experts: stage %d", stage);
+  FMS_REQUIRE(max_tiles > 0 && top > 0 && N > 0 && K > 0 && ldx >= K, "moe_experts: bad sizes tiles=%d top=%d N=%d K=%d ldx=%ld", max_tiles,
+              top, N, K, ldx);
+  ExpertArgs a{x, ldx, w1, w2, y, order, tiles, top, N, K, limit, alpha, shift};
+  const bool mfma = dtype == FMS_BF16 && K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w1 % 16) == 0 &&
+                    (w2 == nullptr || ((uintptr_t)w2 % 16) == 0);
+  const dim3 grid(max_tiles, ceil_div(N, mfma ? TILE_MFMA_COLS : TILE_FMA_COLS));
+  FMS_REQUIRE(grid.y <= 65535, "moe_experts: %d columns are too many for one launch", N);
+  if (dtype == FMS_F32) {
+    if (stage == 0) expert_gate_up_fma_kernel<float><<<grid, TILE_THREADS, 0, stream>>>(a);
+    else expert_down_fma_kernel<float><<<grid, TILE_THREADS, 0, stream>>>(a);
+  } else if (dtype == FMS_BF16) {
+    if (mfma) {
+      if (stage == 0) expert_gate_up_mfma_kernel<<<grid, TILE_THREADS, 0, stream>>>(a);
+      else expert_down_mfma_kernel<<<grid, TILE_THREADS, 0, stream>>>(a);
+    } else {
+      if (stage == 0) expert_gate_up_fma_kernel<bf16><<<grid, TILE_THREADS, 0, stream>>>(a);
+      else expert_down_fma_kernel<bf16><<<grid, TILE_THREADS, 0, stream>>>(a);
+    }
+  } else {
+    FMS_REQUIRE(false, "moe_experts: unknown dtype %d", dtype);
+  }
+  FMS_LAUNCH_CHECK("moe_experts");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// combine
+// --------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+    combine_kernel(const float* __restrict__ y, const float* __restrict__ weights, int top, const T* __restrict__ shared,
+                   const float* __restrict__ shared_gate, long ldg, T* __restrict__ out, int width) {
+  const int t = blockIdx.x;
+  const float sg = shared ? (shared_gate ? 1.f / (1.f + expf(-shared_gate[(size_t)t * ldg])) : 1.f) : 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float v = 0.f;
+    for (int j = 0; j < top; ++j) v = fmaf(weights[(size_t)t * top + j], y[((size_t)t * top + j) * width + i], v);
+    if (shared) v = fmaf(sg, to_f32(shared[(size_t)t * width + i]), v);
+    out[(size_t)t * width + i] = from_f32<T>(v);
+  }
+}
+
+extern "C" int fmsamd_moe_combine(const float* y, const float* weights, int top, const void* shared, const float* shared_gate,
+                                  long ldg, void* out, int dtype, int n_tokens, int width, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  FMS_REQUIRE(n_tokens > 0 && top > 0 && width > 0, "moe_combine: bad sizes T=%d top=%d width=%d", n_tokens, top, width);
+  if (dtype == FMS_F32)
+    combine_kernel<float><<<n_tokens, 256, 0, stream>>>(y, weights, top, (const float*)shared, shared_gate, ldg, (float*)out, width);
+  else if (dtype == FMS_BF16)
+    combine_kernel<bf16><<<n_tokens, 256, 0, stream>>>(y, weights, top, (const bf16*)shared, shared_gate, ldg, (bf16*)out, width);
+  else
+    FMS_REQUIRE(false, "moe_combine: unknown dtype %d", dtype);
+  FMS_LAUNCH_CHECK("moe_combine");
+  return 0;
+}

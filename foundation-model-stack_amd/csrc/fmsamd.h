@@ -6,7 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define FMSAMD_ABI_VERSION 2
+#define FMSAMD_ABI_VERSION 3
 
 // element types
 #define FMS_F32 0
@@ -30,9 +30,9 @@ extern "C" {
 const char* fmsamd_last_error();
 int fmsamd_abi_version();
 
-// resid[t, :] = float(table[ids[t], :])
+// resid[t, :] = float(table[ids[t], :]) * scale
 int fmsamd_embed(const int* ids, const void* table, int table_dtype, float* out, int n_tokens, int width, int vocab,
-                 hipStream_t stream);
+                 float scale, hipStream_t stream);
 
 // resid += branch (float32 sum, written back unless `rows` is given); out = norm(resid) * weight + bias.
 // branch, weight, bias and rows may be null.  act_dtype is the type of branch and out.
@@ -165,6 +165,56 @@ int fmsamd_argmax_static(const float* logits, long ld, int rows, int vocab, int*
 // products instead of 16x16x32.
 int fmsamd_probe_read(const void* buffer, long bytes, int blocks, int contiguous, float* out, hipStream_t stream);
 int fmsamd_probe_mfma(int blocks, int iterations, int large, float* out, double* flops, hipStream_t stream);
+
+// ---- norms behind a branch, further activations (norm_chain.hip) ----------------------------------------------
+// resid += branch / rms(branch) * branch_weight (float32, written back unless `rows` is given);
+// out = resid / rms(resid) * weight (out null: the sum only).  Both weights have weight_dtype; either may be null.
+int fmsamd_norm_add_norm(float* resid, const void* branch, int act_dtype, const void* branch_weight, float branch_eps,
+                         const void* weight, int weight_dtype, float eps, void* out, const int* rows, int n_out, int width,
+                         hipStream_t stream);
+// out[t, 0:n] = x[t, col0 : col0 + n] / rms * weight for float32 rows ldx apart
+int fmsamd_rms_norm_cols(const float* x, long ldx, int col0, int n, const void* weight, int weight_dtype, float eps,
+                         void* out, int out_dtype, long ldo, int rows, hipStream_t stream);
+// out = act(x), act one of FMS_ACT_*
+int fmsamd_activate(const void* x, void* out, int dtype, long n, int act, hipStream_t stream);
+// gu [T, 2 * hidden] (gate first): out = g' sigmoid(alpha g') (u' + shift), g' = min(g, limit), u' = clamp(u, +-limit)
+int fmsamd_clamped_gated_act(const void* gu, void* out, int dtype, int n_tokens, int hidden, float limit, float alpha,
+                             float shift, hipStream_t stream);
+
+// ---- attention over a latent cache (latent_attention.hip) ---------------------------------------------------------
+// The cache holds one row [rank + rot] per token: pages [page][token in page][rank + rot].
+// down: float32 rows whose columns col0 .. col0 + rank + rot are the latent before its norm and the shared key part
+// before its rotation; the normed latent and the rotated part are written into the token's page.
+int fmsamd_latent_kv_write(const float* down, long ld, int col0, int rank, int rot, const void* norm_weight,
+                           int weight_dtype, float eps, const int* positions, const int* seq_of_token,
+                           const int* block_table, int table_stride, const float* cos_t, const float* sin_t, int max_pos,
+                           void* cache, int cache_dtype, int n_tokens, hipStream_t stream);
+// qa[t, h, rank : rank + rot] = rotate(q[t, h, dim : dim + rot]); q rows hold nheads x (dim + rot), qa rows nheads x (rank + rot)
+int fmsamd_latent_q_rotate(const void* q, long ldq, int dtype, int nheads, int dim, int rot, void* qa, long ldqa, int rank,
+                           const int* positions, const float* cos_t, const float* sin_t, int max_pos, int n_tokens,
+                           hipStream_t stream);
+// y[t, h, 0:N] = W[h] x[t, h, 0:K] (W [nheads, N, K]), times sigmoid(gate[t * ldg + h]) if gate is given
+int fmsamd_headwise_linear(const void* x, long ldx, long x_head_stride, const void* w, void* y, long ldy,
+                           long y_head_stride, const float* gate, long ldg, int dtype, int n_tokens, int nheads, int N,
+                           int K, hipStream_t stream);
+// out[t, h, 0:rank] = sum_j p_j cache[j, 0:rank], p = softmax over the visible keys j (and the sink, if given: float32
+// [nheads], unscaled, in the denominator only) of scale * qa[t, h, :] . cache[j, :]
+int fmsamd_latent_attn_generic(const void* qa, long ldq, void* out, long ldo, int dtype, const int* positions,
+                               const int* seq_of_token, const int* block_table, int table_stride, const void* cache,
+                               const float* sink, int n_tokens, int nheads, int rank, int rot, float scale, int window,
+                               hipStream_t stream);
+
+// ---- experts (experts.hip) -----------------------------------------------------------------------------------------
+int fmsamd_moe_route(const float* logits, long ld, int n_tokens, int n_experts, int top, int* ids, float* weights,
+                     hipStream_t stream);
+int fmsamd_moe_max_tiles(int n_pairs, int n_experts);
+// order [n_pairs], tiles [max_tiles][3] = (expert, first row in order, rows)
+int fmsamd_moe_group(const int* ids, int n_pairs, int n_experts, int* order, int* tiles, int max_tiles, hipStream_t stream);
+int fmsamd_moe_experts(int stage, const void* x, long ldx, const void* w1, const void* w2, void* y, int dtype,
+                       const int* order, const int* tiles, int max_tiles, int top, int N, int K, float limit, float alpha,
+                       float shift, hipStream_t stream);
+int fmsamd_moe_combine(const float* y, const float* weights, int top, const void* shared, const float* shared_gate, long ldg,
+                       void* out, int dtype, int n_tokens, int width, hipStream_t stream);
 
 #ifdef __cplusplus
 }

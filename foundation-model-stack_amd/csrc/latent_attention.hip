@@ -1,0 +1,300 @@
+// Attention over a latent cache: every token leaves one row [latent (R) | rotated shared key part (P)] in the
+// cache, and all query heads read that one row.  With per-head matrices Uk [D, R] (keys) and Uv [V, R] (values)
+//   score(t, j, h) = (q_plain . Uk_h c_j + q_rot . k_rot_j) * scale = ((Uk_h^T q_plain) . c_j + q_rot . k_rot_j) * scale
+//   out(t, h)      = Uv_h sum_j p_j c_j
+// so the kernels never expand keys or values: the query goes into the latent space once per token and head, attention
+// runs as one shared "kv head" with keys of R + P and values of R elements (the first R of the same row), and the
+// result leaves the latent space once per token and head.  Whole prompts, portions and single tokens run the same way.
+//
+// The softmax may have a sink: a learned logit per head that counts once in the denominator and has no value.  It is
+// the state in which the running maximum and sum start.
+//
+//   latent_kv_write:      RMS norm of the latent, rotation of the shared key part, row written into its page
+//   latent_q_rotate:      the rotated part of every head's query into its place behind the latent part
+//   headwise_linear:      y[t, h, :] = W_h x[t, h, :] (optionally times sigmoid(gate[t, h])), FMA or MFMA
+//   latent_attn_generic:  float32 arithmetic on any storage type; one block per (head, token)
+//   latent_attn_mfma:     bfloat16, a block per 16 (token, head) rows ... see below
+//
+// Cache layout: rows [page][token in page][R + P].
+#include "common.h"
+#include "fmsamd.h"
+#include "tile_product.h"
+
+// --------------------------------------------------------------------------
+// cache write
+// --------------------------------------------------------------------------
+template <typename CT>
+__global__ void __launch_bounds__(256)
+    latent_kv_write_kernel(const float* __restrict__ down, long ld, int col0, int rank, int rot, const void* __restrict__ w,
+                           int w_dtype, float eps, const int* __restrict__ positions, const int* __restrict__ seq_of_token,
+                           const int* __restrict__ block_table, int table_stride, const float* __restrict__ cos_t,
+                           const float* __restrict__ sin_t, CT* __restrict__ cache) {
+  __shared__ float scratch[17];
+  const int t = blockIdx.x;
+  const int seq = seq_of_token[t];
+  if (seq < 0) return;
+  const int pos = positions[t];
+  const int page = block_table[(size_t)seq * table_stride + pos / PAGE_TOKENS];
+  if (page < 0) return;
+  const float* x = down + (size_t)t * ld + col0;
+  CT* row = cache + ((size_t)page * PAGE_TOKENS + pos % PAGE_TOKENS) * (rank + rot);
+  float sq = 0.f;
+  for (int i = threadIdx.x; i < rank; i += blockDim.x) sq = fmaf(x[i], x[i], sq);
+  const float rs = rsqrtf(block_sum(sq, scratch) / (float)rank + eps);
+  for (int i = threadIdx.x; i < rank; i += blockDim.x) {
+    const float wi = w == nullptr ? 1.f : (w_dtype == FMS_F32 ? ((const float*)w)[i] : (float)((const bf16*)w)[i]);
+    row[i] = from_f32<CT>(x[i] * rs * wi);
+  }
+  const int half = rot / 2;
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    const float c = cos_t[(size_t)pos * half + i], s = sin_t[(size_t)pos * half + i];
+    const float u = x[rank + 2 * i], v = x[rank + 2 * i + 1];
+    row[rank + 2 * i] = from_f32<CT>(u * c - v * s);
+    row[rank + 2 * i + 1] = from_f32<CT>(v * c + u * s);
+  }
+}
+
+extern "C" int fmsamd_latent_kv_write(const float* down, long ld, int col0, int rank, int rot, const void* norm_weight,
+                                      int weight_dtype, float eps, const int* positions, const int* seq_of_token,
+                                      const int* block_table, int table_stride, const float* cos_t, const float* sin_t,
+                                      int max_pos, void* cache, int cache_dtype, int n_tokens, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  FMS_REQUIRE(n_tokens > 0 && rank > 0 && rot >= 0 && rot % 2 == 0 && col0 >= 0 && ld >= col0 + rank + rot,
+              "latent_kv_write: bad sizes T=%d rank=%d rot=%d col0=%d ld=%ld", n_tokens, rank, rot, col0, ld);
+  FMS_REQUIRE(rot == 0 || (cos_t != nullptr && sin_t != nullptr && max_pos > 0), "latent_kv_write: a rotation needs its tables");
+  if (cache_dtype == FMS_F32)
+    latent_kv_write_kernel<float><<<n_tokens, 256, 0, stream>>>(down, ld, col0, rank, rot, norm_weight, weight_dtype, eps,
+                                                                positions, seq_of_token, block_table, table_stride, cos_t,
+                                                                sin_t, (float*)cache);
+  else if (cache_dtype == FMS_BF16)
+    latent_kv_write_kernel<bf16><<<n_tokens, 256, 0, stream>>>(down, ld, col0, rank, rot, norm_weight, weight_dtype, eps,
+                                                               positions, seq_of_token, block_table, table_stride, cos_t,
+                                                               sin_t, (bf16*)cache);
+  else
+    FMS_REQUIRE(false, "latent_kv_write: unknown dtype %d", cache_dtype);
+  FMS_LAUNCH_CHECK("latent_kv_write");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// queries: q [T, H, D + P] -> qa[t, h, R : R + P] = rotate(q[t, h, D : D + P])
+// --------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+    latent_q_rotate_kernel(const T* __restrict__ q, long ldq, int nheads, int dim, int rot, T* __restrict__ qa, long ldqa,
+                           int rank, const int* __restrict__ positions, const float* __restrict__ cos_t,
+                           const float* __restrict__ sin_t) {
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  const int half = rot / 2;
+  for (int i = threadIdx.x; i < nheads * half; i += blockDim.x) {
+    const int h = i / half, p = i % half;
+    const T* src = q + (size_t)t * ldq + (size_t)h * (dim + rot) + dim + 2 * p;
+    T* dst = qa + (size_t)t * ldqa + (size_t)h * (rank + rot) + rank + 2 * p;
+    const float c = cos_t[(size_t)pos * half + p], s = sin_t[(size_t)pos * half + p];
+    const float u = to_f32(src[0]), v = to_f32(src[1]);
+    dst[0] = from_f32<T>(u * c - v * s);
+    dst[1] = from_f32<T>(v * c + u * s);
+  }
+}
+
+extern "C" int fmsamd_latent_q_rotate(const void* q, long ldq, int dtype, int nheads, int dim, int rot, void* qa, long ldqa,
+                                      int rank, const int* positions, const float* cos_t, const float* sin_t, int max_pos,
+                                      int n_tokens, hipStream_t stream) {
+  if (n_tokens == 0 || rot == 0) return 0;
+  FMS_REQUIRE(n_tokens > 0 && nheads > 0 && dim >= 0 && rot > 0 && rot % 2 == 0 && rank > 0, "latent_q_rotate: bad sizes");
+  FMS_REQUIRE(ldq >= (long)nheads * (dim + rot) && ldqa >= (long)nheads * (rank + rot), "latent_q_rotate: rows too short");
+  FMS_REQUIRE(cos_t != nullptr && sin_t != nullptr && max_pos > 0, "latent_q_rotate: a rotation needs its tables");
+  if (dtype == FMS_F32)
+    latent_q_rotate_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)q, ldq, nheads, dim, rot, (float*)qa, ldqa, rank,
+                                                                positions, cos_t, sin_t);
+  else if (dtype == FMS_BF16)
+    latent_q_rotate_kernel<bf16><<<n_tokens, 256, 0, stream>>>((const bf16*)q, ldq, nheads, dim, rot, (bf16*)qa, ldqa, rank,
+                                                               positions, cos_t, sin_t);
+  else
+    FMS_REQUIRE(false, "latent_q_rotate: unknown dtype %d", dtype);
+  FMS_LAUNCH_CHECK("latent_q_rotate");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// y[t, h, n] = sum_k x[t, h, k] W[h, n, k]  (* sigmoid(gate[t, h]))
+// --------------------------------------------------------------------------
+struct HeadwiseArgs {
+  const void* x;
+  long ldx, xs;  // row stride, head stride of x (elements)
+  const void* w;  // [H, N, K]
+  void* y;
+  long ldy, ys;
+  const float* gate;  // logits [T, ldg] or null
+  long ldg;
+  int T, H, N, K;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(TILE_THREADS) headwise_fma_kernel(HeadwiseArgs a) {
+  const int t0 = blockIdx.x * TILE_ROWS, h = blockIdx.y, n0 = blockIdx.z * TILE_FMA_COLS;
+  const T* x = (const T*)a.x + (size_t)h * a.xs;
+  const T* w = (const T*)a.w + (size_t)h * a.N * a.K;
+  float acc[4];
+  tile_product_fma<T>([&](int m) { return t0 + m < a.T ? x + (size_t)(t0 + m) * a.ldx : (const T*)nullptr; },
+                      [&](int n) { return n0 + n < a.N ? w + (size_t)(n0 + n) * a.K : (const T*)nullptr; }, a.K, acc);
+  const int n = n0 + threadIdx.x % 64;
+  if (n >= a.N) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int t = t0 + (threadIdx.x / 64) * 4 + i;
+    if (t < a.T) {
+      float v = acc[i];
+      if (a.gate) v *= 1.f / (1.f + expf(-a.gate[(size_t)t * a.ldg + h]));
+      ((T*)a.y)[(size_t)t * a.ldy + (size_t)h * a.ys + n] = from_f32<T>(v);
+    }
+  }
+}
+
+__global__ void __launch_bounds__(TILE_THREADS) headwise_mfma_kernel(HeadwiseArgs a) {
+  const int t0 = blockIdx.x * TILE_ROWS, h = blockIdx.y, n0 = blockIdx.z * TILE_MFMA_COLS;
+  const bf16* x = (const bf16*)a.x + (size_t)h * a.xs;
+  const bf16* w = (const bf16*)a.w + (size_t)h * a.N * a.K;
+  f32x4 acc[4];
+  tile_product_mfma([&](int m) { return t0 + m < a.T ? x + (size_t)(t0 + m) * a.ldx : (const bf16*)nullptr; },
+                    [&](int n) { return n0 + n < a.N ? w + (size_t)(n0 + n) * a.K : (const bf16*)nullptr; }, a.K, acc);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int t = t0 + (lane >> 4) * 4 + i;
+    if (t >= a.T) continue;
+    const float g = a.gate ? 1.f / (1.f + expf(-a.gate[(size_t)t * a.ldg + h])) : 1.f;
+#pragma unroll
+    for (int tl = 0; tl < 4; ++tl) {
+      const int n = n0 + wave * 64 + tl * 16 + (lane & 15);
+      if (n < a.N) ((bf16*)a.y)[(size_t)t * a.ldy + (size_t)h * a.ys + n] = (bf16)(acc[tl][i] * g);
+    }
+  }
+}
+
+extern "C" int fmsamd_headwise_linear(const void* x, long ldx, long x_head_stride, const void* w, void* y, long ldy,
+                                      long y_head_stride, const float* gate, long ldg, int dtype, int n_tokens, int nheads,
+                                      int N, int K, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  FMS_REQUIRE(n_tokens > 0 && nheads > 0 && nheads <= 65535 && N > 0 && K > 0, "headwise_linear: bad sizes T=%d H=%d N=%d K=%d",
+              n_tokens, nheads, N, K);
+  FMS_REQUIRE(ldx >= (nheads - 1) * x_head_stride + K && ldy >= (nheads - 1) * y_head_stride + N,
+              "headwise_linear: rows too short for %d heads", nheads);
+  HeadwiseArgs a{x, ldx, x_head_stride, w, y, ldy, y_head_stride, gate, ldg, n_tokens, nheads, N, K};
+  const int row_tiles = ceil_div(n_tokens, TILE_ROWS);
+  if (dtype == FMS_F32) {
+    headwise_fma_kernel<float><<<dim3(row_tiles, nheads, ceil_div(N, TILE_FMA_COLS)), TILE_THREADS, 0, stream>>>(a);
+  } else if (dtype == FMS_BF16) {
+    const bool aligned = K % 8 == 0 && ldx % 8 == 0 && x_head_stride % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0;
+    if (aligned)
+      headwise_mfma_kernel<<<dim3(row_tiles, nheads, ceil_div(N, TILE_MFMA_COLS)), TILE_THREADS, 0, stream>>>(a);
+    else
+      headwise_fma_kernel<bf16><<<dim3(row_tiles, nheads, ceil_div(N, TILE_FMA_COLS)), TILE_THREADS, 0, stream>>>(a);
+  } else {
+    FMS_REQUIRE(false, "headwise_linear: unknown dtype %d", dtype);
+  }
+  FMS_LAUNCH_CHECK("headwise_linear");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// generic attention: one block per (head, token), keys 256 at a time
+// --------------------------------------------------------------------------
+#define LAT_THREADS 256
+#define LAT_MAX_RANK 1024  // 4 output elements a thread
+
+template <typename T>
+__global__ void __launch_bounds__(LAT_THREADS)
+    latent_attn_generic_kernel(const T* __restrict__ qa, long ldq, T* __restrict__ out, long ldo,
+                               const int* __restrict__ positions, const int* __restrict__ seq_of_token,
+                               const int* __restrict__ block_table, int table_stride, const T* __restrict__ cache,
+                               const float* __restrict__ sink, int rank, int rot, float scale, int window) {
+  extern __shared__ float qs[];  // rank + rot
+  __shared__ float ps[LAT_THREADS];
+  __shared__ float scratch[17];
+  const int h = blockIdx.x, t = blockIdx.y;
+  const int width = rank + rot;
+  const int seq = seq_of_token[t];
+  T* o = out + (size_t)t * ldo + (size_t)h * rank;
+  if (seq < 0) {
+    for (int d = threadIdx.x; d < rank; d += blockDim.x) o[d] = from_f32<T>(0.f);
+    return;
+  }
+  const int pos = positions[t];
+  const int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
+  const int* bt = block_table + (size_t)seq * table_stride;
+  const T* qrow = qa + (size_t)t * ldq + (size_t)h * width;
+  for (int d = threadIdx.x; d < width; d += blockDim.x) qs[d] = to_f32(qrow[d]);
+  __syncthreads();
+
+  // the sink is where the softmax starts: a logit that is already in the denominator, with no value
+  float m_run = sink ? sink[h] : -1e30f, l_run = sink ? 1.f : 0.f;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  const int first = lo - lo % PAGE_TOKENS;  // chunks begin at a page's first token
+  for (int base = first; base <= pos; base += LAT_THREADS) {
+    const int j = base + threadIdx.x;
+    float s = -INFINITY;
+    if (j >= lo && j <= pos) {
+      const T* krow = cache + (readable_page(bt[j / PAGE_TOKENS]) * PAGE_TOKENS + j % PAGE_TOKENS) * width;
+      float dot = 0.f;
+      for (int d = 0; d < width; ++d) dot = fmaf(qs[d], to_f32(krow[d]), dot);
+      s = dot * scale;
+    }
+    const float m_new = fmaxf(m_run, block_max(s, scratch));
+    const float p = (j >= lo && j <= pos) ? expf(s - m_new) : 0.f;
+    const float alpha = expf(m_run - m_new);
+    ps[threadIdx.x] = p;
+    const float psum = block_sum(p, scratch);  // has the barriers that publish ps
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] *= alpha;
+    const int n = pos - base + 1 < LAT_THREADS ? pos - base + 1 : LAT_THREADS;
+    for (int pg = 0; pg * PAGE_TOKENS < n; ++pg) {
+      const T* prow = cache + readable_page(bt[base / PAGE_TOKENS + pg]) * PAGE_TOKENS * width;
+      const int cnt = n - pg * PAGE_TOKENS < PAGE_TOKENS ? n - pg * PAGE_TOKENS : PAGE_TOKENS;
+      for (int i = 0; i < cnt; ++i) {
+        const float pi = ps[pg * PAGE_TOKENS + i];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int d = threadIdx.x + e * LAT_THREADS;
+          if (d < rank) acc[e] = fmaf(pi, to_f32(prow[(size_t)i * width + d]), acc[e]);
+        }
+      }
+    }
+    __syncthreads();  // ps is overwritten by the next chunk
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int d = threadIdx.x + e * LAT_THREADS;
+    if (d < rank) o[d] = from_f32<T>(l_run > 0.f ? acc[e] / l_run : 0.f);
+  }
+}
+
+extern "C" int fmsamd_latent_attn_generic(const void* qa, long ldq, void* out, long ldo, int dtype, const int* positions,
+                                          const int* seq_of_token, const int* block_table, int table_stride,
+                                          const void* cache, const float* sink, int n_tokens, int nheads, int rank, int rot,
+                                          float scale, int window, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  FMS_REQUIRE(n_tokens > 0 && n_tokens <= 65535 && nheads > 0, "latent_attn_generic: %d tokens, %d heads (at most 65535 tokens a launch)",
+              n_tokens, nheads);
+  FMS_REQUIRE(rank > 0 && rank <= LAT_MAX_RANK && rot >= 0 && rank + rot <= 2048, "latent_attn_generic: latent size %d (at most %d), rotated size %d",
+              rank, LAT_MAX_RANK, rot);
+  FMS_REQUIRE(ldq >= (long)nheads * (rank + rot) && ldo >= (long)nheads * rank, "latent_attn_generic: rows too short");
+  FMS_REQUIRE(window >= 0, "latent_attn_generic: window %d", window);
+  const dim3 grid(nheads, n_tokens);
+  const size_t lds = (size_t)(rank + rot) * sizeof(float);
+  if (dtype == FMS_F32)
+    latent_attn_generic_kernel<float><<<grid, LAT_THREADS, lds, stream>>>((const float*)qa, ldq, (float*)out, ldo, positions,
+                                                                          seq_of_token, block_table, table_stride,
+                                                                          (const float*)cache, sink, rank, rot, scale, window);
+  else if (dtype == FMS_BF16)
+    latent_attn_generic_kernel<bf16><<<grid, LAT_THREADS, lds, stream>>>((const bf16*)qa, ldq, (bf16*)out, ldo, positions,
+                                                                         seq_of_token, block_table, table_stride,
+                                                                         (const bf16*)cache, sink, rank, rot, scale, window);
+  else
+    FMS_REQUIRE(false, "latent_attn_generic: unknown dtype %d", dtype);
+  FMS_LAUNCH_CHECK("latent_attn_generic");
+  return 0;
+}

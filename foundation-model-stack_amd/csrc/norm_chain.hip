@@ -1,0 +1,146 @@
+// Norms that sit behind a branch, and activations of feed-forwards that are not "act(gate) * up".
+//
+//   norm_add_norm: a block whose branches are normed before they join the stream,
+//       stream += branch / rms(branch) * wb;   out = stream / rms(stream) * w
+//     in one pass over the row: two row norms and the residual sum, all float32.
+//   rms_norm_cols: the RMS norm of a run of columns of float32 rows (a slice of a fused projection).
+//   activate: out = act(x), the activations of common.h.
+//   clamped_gated_act: out = g' * sigmoid(alpha g') * (u' + shift), g' = min(g, limit), u' = clamp(u, -limit, limit).
+#include "common.h"
+#include "fmsamd.h"
+
+__device__ __forceinline__ float load_scale(const void* w, int dtype, int i) {
+  if (w == nullptr) return 1.f;
+  return dtype == FMS_F32 ? ((const float*)w)[i] : (float)((const bf16*)w)[i];
+}
+
+// One block per output row; the row waits in LDS (width floats) between the two reductions.
+template <typename T>
+__global__ void __launch_bounds__(256)
+    norm_add_norm_kernel(float* __restrict__ resid, const T* __restrict__ branch, const void* __restrict__ wb, float eps_b,
+                         const void* __restrict__ w, int w_dtype, float eps, T* __restrict__ out,
+                         const int* __restrict__ rows, int width) {
+  extern __shared__ float row[];
+  __shared__ float scratch[17];
+  const int r = rows ? rows[blockIdx.x] : blockIdx.x;
+  float* x = resid + (size_t)r * width;
+  const T* b = branch + (size_t)r * width;
+  float sq = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float v = to_f32(b[i]);
+    row[i] = v;
+    sq = fmaf(v, v, sq);
+  }
+  const float rb = rsqrtf(block_sum(sq, scratch) / (float)width + eps_b);
+  sq = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float v = x[i] + row[i] * rb * load_scale(wb, w_dtype, i);
+    row[i] = v;
+    if (!rows) x[i] = v;
+    sq = fmaf(v, v, sq);
+  }
+  if (out == nullptr) return;
+  const float rs = rsqrtf(block_sum(sq, scratch) / (float)width + eps);
+  T* o = out + (size_t)blockIdx.x * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = from_f32<T>(row[i] * rs * load_scale(w, w_dtype, i));
+}
+
+extern "C" int fmsamd_norm_add_norm(float* resid, const void* branch, int act_dtype, const void* branch_weight,
+                                    float branch_eps, const void* weight, int weight_dtype, float eps, void* out,
+                                    const int* rows, int n_out, int width, hipStream_t stream) {
+  if (n_out == 0) return 0;
+  FMS_REQUIRE(n_out > 0 && width > 0 && width <= 16384, "norm_add_norm: bad sizes rows=%d width=%d", n_out, width);
+  FMS_REQUIRE(resid != nullptr && branch != nullptr, "norm_add_norm: the stream and the branch are needed");
+  const size_t lds = (size_t)width * sizeof(float);
+  if (act_dtype == FMS_F32)
+    norm_add_norm_kernel<float><<<n_out, 256, lds, stream>>>(resid, (const float*)branch, branch_weight, branch_eps,
+                                                             weight, weight_dtype, eps, (float*)out, rows, width);
+  else if (act_dtype == FMS_BF16)
+    norm_add_norm_kernel<bf16><<<n_out, 256, lds, stream>>>(resid, (const bf16*)branch, branch_weight, branch_eps,
+                                                            weight, weight_dtype, eps, (bf16*)out, rows, width);
+  else
+    FMS_REQUIRE(false, "norm_add_norm: unknown dtype %d", act_dtype);
+  FMS_LAUNCH_CHECK("norm_add_norm");
+  return 0;
+}
+
+// out[t, 0:n] = x[t, col0 : col0 + n] / rms * w, x float32 with rows ldx apart
+template <typename T>
+__global__ void __launch_bounds__(256)
+    rms_norm_cols_kernel(const float* __restrict__ x, long ldx, int col0, int n, const void* __restrict__ w, int w_dtype,
+                         float eps, T* __restrict__ out, long ldo) {
+  __shared__ float scratch[17];
+  const float* xr = x + (size_t)blockIdx.x * ldx + col0;
+  float sq = 0.f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) sq = fmaf(xr[i], xr[i], sq);
+  const float rs = rsqrtf(block_sum(sq, scratch) / (float)n + eps);
+  T* o = out + (size_t)blockIdx.x * ldo;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) o[i] = from_f32<T>(xr[i] * rs * load_scale(w, w_dtype, i));
+}
+
+extern "C" int fmsamd_rms_norm_cols(const float* x, long ldx, int col0, int n, const void* weight, int weight_dtype,
+                                    float eps, void* out, int out_dtype, long ldo, int rows, hipStream_t stream) {
+  if (rows == 0) return 0;
+  FMS_REQUIRE(rows > 0 && n > 0 && col0 >= 0 && ldx >= col0 + n && ldo >= n, "rms_norm_cols: bad sizes rows=%d n=%d col0=%d ldx=%ld",
+              rows, n, col0, ldx);
+  if (out_dtype == FMS_F32)
+    rms_norm_cols_kernel<float><<<rows, 256, 0, stream>>>(x, ldx, col0, n, weight, weight_dtype, eps, (float*)out, ldo);
+  else if (out_dtype == FMS_BF16)
+    rms_norm_cols_kernel<bf16><<<rows, 256, 0, stream>>>(x, ldx, col0, n, weight, weight_dtype, eps, (bf16*)out, ldo);
+  else
+    FMS_REQUIRE(false, "rms_norm_cols: unknown dtype %d", out_dtype);
+  FMS_LAUNCH_CHECK("rms_norm_cols");
+  return 0;
+}
+
+template <typename T>
+__global__ void activate_kernel(const T* __restrict__ x, T* __restrict__ out, long n, int act) {
+  const long stride = (long)gridDim.x * blockDim.x;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+    out[i] = from_f32<T>(fms_activate(to_f32(x[i]), act));
+}
+
+extern "C" int fmsamd_activate(const void* x, void* out, int dtype, long n, int act, hipStream_t stream) {
+  if (n == 0) return 0;
+  FMS_REQUIRE(n > 0 && act >= 0 && act <= FMS_ACT_LAST, "activate: bad arguments n=%ld act=%d", n, act);
+  const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+  if (dtype == FMS_F32)
+    activate_kernel<float><<<blocks, 256, 0, stream>>>((const float*)x, (float*)out, n, act);
+  else if (dtype == FMS_BF16)
+    activate_kernel<bf16><<<blocks, 256, 0, stream>>>((const bf16*)x, (bf16*)out, n, act);
+  else
+    FMS_REQUIRE(false, "activate: unknown dtype %d", dtype);
+  FMS_LAUNCH_CHECK("activate");
+  return 0;
+}
+
+__device__ __forceinline__ float clamped_gate(float g, float u, float limit, float alpha, float shift) {
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  return g / (1.f + expf(-alpha * g)) * (u + shift);
+}
+
+// gu [T, 2 * hidden] (gate first), out [T, hidden]
+template <typename T>
+__global__ void clamped_gated_act_kernel(const T* __restrict__ gu, T* __restrict__ out, int hidden, float limit,
+                                         float alpha, float shift) {
+  const T* g = gu + (size_t)blockIdx.x * 2 * hidden;
+  T* o = out + (size_t)blockIdx.x * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x)
+    o[i] = from_f32<T>(clamped_gate(to_f32(g[i]), to_f32(g[hidden + i]), limit, alpha, shift));
+}
+
+extern "C" int fmsamd_clamped_gated_act(const void* gu, void* out, int dtype, int n_tokens, int hidden, float limit,
+                                        float alpha, float shift, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  FMS_REQUIRE(n_tokens > 0 && hidden > 0 && limit > 0.f, "clamped_gated_act: bad arguments T=%d hidden=%d limit=%g", n_tokens,
+              hidden, (double)limit);
+  if (dtype == FMS_F32)
+    clamped_gated_act_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)gu, (float*)out, hidden, limit, alpha, shift);
+  else if (dtype == FMS_BF16)
+    clamped_gated_act_kernel<bf16><<<n_tokens, 256, 0, stream>>>((const bf16*)gu, (bf16*)out, hidden, limit, alpha, shift);
+  else
+    FMS_REQUIRE(false, "clamped_gated_act: unknown dtype %d", dtype);
+  FMS_LAUNCH_CHECK("clamped_gated_act");
+  return 0;
+}

@@ -26,7 +26,9 @@ class DecoderModel(Part):
         for i, layer in enumerate(spec.layers):
             pos = self.positions[layer.position] if layer.position is not None else None
             mixer = make_part("mixer", layer.mixer.kind, width=spec.width, position_encoder=pos, **layer.mixer.args)
-            ff = make_part("feed_forward", layer.feed_forward.kind, width=spec.width, **layer.feed_forward.args)
+            ff = None  # a layer may have no feed-forward, if its block takes None
+            if layer.feed_forward is not None:
+                ff = make_part("feed_forward", layer.feed_forward.kind, width=spec.width, **layer.feed_forward.args)
             # a block names the norms it wants as constructor arguments (none, two, four ...); each is built from the
             # layer's list of norm specs, or from its one norm spec for all of them
             wanted = part_attribute("block", layer.block.kind, "norm_arguments", ("norm1", "norm2"))

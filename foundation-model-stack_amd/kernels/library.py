@@ -17,7 +17,7 @@ import torch  # noqa: F401  (loads libamdhip64 before our library asks for it)
 
 from . import build as _build
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _lib: Optional[ctypes.CDLL] = None
 _lock = threading.Lock()
@@ -25,7 +25,7 @@ _lock = threading.Lock()
 P, I, L, F = c_void_p, c_int, c_long, c_float
 
 _SIGNATURES = {
-    "fmsamd_embed": [P, P, I, P, I, I, I, P],
+    "fmsamd_embed": [P, P, I, P, I, I, I, F, P],
     "fmsamd_add_norm": [P, P, I, P, P, I, P, P, I, I, F, I, P],
     "fmsamd_gated_act": [P, P, I, P, I, I, I, I, P],
     "fmsamd_cast": [P, I, P, I, L, P],
@@ -47,6 +47,18 @@ _SIGNATURES = {
     "fmsamd_gemm_skinny_residual_bf16": [P, L, P, P, I, P, L, P, I, P, L, P, I, I, I, I, P, P, L, P],
     "fmsamd_sample": [P, L, I, I, I, F, I, P, P, P],
     "fmsamd_argmax": [P, L, I, I, P, L, P, P],
+    "fmsamd_norm_add_norm": [P, P, I, P, F, P, I, F, P, P, I, I, P],
+    "fmsamd_rms_norm_cols": [P, L, I, I, P, I, F, P, I, L, I, P],
+    "fmsamd_activate": [P, P, I, L, I, P],
+    "fmsamd_clamped_gated_act": [P, P, I, I, I, F, F, F, P],
+    "fmsamd_latent_kv_write": [P, L, I, I, I, P, I, F, P, P, P, I, P, P, I, P, I, I, P],
+    "fmsamd_latent_q_rotate": [P, L, I, I, I, I, P, L, I, P, P, P, I, I, P],
+    "fmsamd_headwise_linear": [P, L, L, P, P, L, L, P, L, I, I, I, I, I, P],
+    "fmsamd_latent_attn_generic": [P, L, P, L, I, P, P, P, I, P, P, I, I, I, I, F, I, P],
+    "fmsamd_moe_route": [P, L, I, I, I, P, P, P],
+    "fmsamd_moe_group": [P, I, I, P, P, I, P],
+    "fmsamd_moe_experts": [I, P, L, P, P, P, I, P, P, I, I, I, I, F, F, F, P],
+    "fmsamd_moe_combine": [P, P, I, P, P, L, P, I, I, I, P],
     "fmsamd_probe_read": [P, L, I, I, P, P],
     "fmsamd_probe_mfma": [I, I, I, P, P, P],
 }
@@ -86,6 +98,8 @@ def load(verbose: bool = True) -> ctypes.CDLL:
             fn.restype = c_int
         lib.fmsamd_attn_prefill_qblock.restype = c_int
         lib.fmsamd_attn_prefill_qblock.argtypes = [I, I, I, I]
+        lib.fmsamd_moe_max_tiles.restype = c_int
+        lib.fmsamd_moe_max_tiles.argtypes = [I, I]
         lib.fmsamd_argmax_workspace.restype = c_long
         lib.fmsamd_argmax_workspace.argtypes = [I, I]
         lib.fmsamd_attn_decode_workspace.restype = c_long

@@ -57,15 +57,15 @@ def _rows2d(name: str, t: torch.Tensor) -> None:
 
 
 # --------------------------------------------------------------------------
-def embed(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
-    """float32 rows of `table` for int32 `ids` [T] -> [T, width]."""
+def embed(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """float32 rows of `table` for int32 `ids` [T], times `scale` -> [T, width]."""
     _need_cuda(ids, table)
     _need_i32("ids", ids)
     if table.dim() != 2 or not table.is_contiguous():
         raise ValueError("embedding table must be a contiguous [vocab, width] tensor")
     out = torch.empty(ids.numel(), table.shape[1], dtype=torch.float32, device=table.device)
     check(load().fmsamd_embed(ids.data_ptr(), table.data_ptr(), _code(table.dtype), out.data_ptr(), ids.numel(),
-                              table.shape[1], table.shape[0], _stream()))
+                              table.shape[1], table.shape[0], float(scale), _stream()))
     return out
 
 
@@ -586,6 +586,258 @@ def gated_linear(
         raise ValueError(f"a deferred row norm goes with the bfloat16 product of at most {SKINNY_FAST_ROWS} rows")
     gu = linear(x, weight, None, allow_library=allow_library)
     return gated_act(gu, bias, activation)
+
+
+# --------------------------------------------------------------------------
+# norms behind a branch, further activations
+# --------------------------------------------------------------------------
+def norm_add_norm(
+    resid: torch.Tensor,
+    branch: torch.Tensor,
+    branch_weight: Optional[torch.Tensor],
+    branch_eps: float,
+    weight: Optional[torch.Tensor],
+    eps: float,
+    out_dtype: torch.dtype,
+    rows: Optional[torch.Tensor] = None,
+    want_out: bool = True,
+) -> Optional[torch.Tensor]:
+    """resid += branch / rms(branch) * branch_weight (float32, in place unless `rows` is given); returns
+    resid / rms(resid) * weight in `out_dtype` (only `rows` if given; None if want_out is False)."""
+    _need_cuda(resid, branch, branch_weight, weight, rows)
+    if resid.dtype != torch.float32 or resid.dim() != 2 or not resid.is_contiguous():
+        raise ValueError("the residual stream must be a contiguous float32 [T, width] tensor")
+    T, width = resid.shape
+    if branch.shape != resid.shape or not branch.is_contiguous() or branch.dtype != out_dtype:
+        raise ValueError(f"branch must be contiguous {tuple(resid.shape)} of {out_dtype}, got {tuple(branch.shape)} {branch.dtype}")
+    wdtype = None
+    for name, t in (("branch weight", branch_weight), ("weight", weight)):
+        if t is not None:
+            if t.shape != (width,) or not t.is_contiguous():
+                raise ValueError(f"norm {name} must be a contiguous [{width}] tensor, got {tuple(t.shape)}")
+            if wdtype is not None and t.dtype != wdtype:
+                raise TypeError("the two norm weights must have one dtype")
+            wdtype = t.dtype
+    if width > 16384:
+        raise ValueError(f"norm_add_norm keeps a row of at most 16384 elements, the width is {width}")
+    n_out = T
+    if rows is not None:
+        _need_i32("rows", rows)
+        n_out = rows.numel()
+    out = torch.empty(n_out, width, dtype=out_dtype, device=resid.device) if want_out else None
+    check(load().fmsamd_norm_add_norm(resid.data_ptr(), branch.data_ptr(), _code(out_dtype), _ptr(branch_weight), float(branch_eps),
+                                      _ptr(weight), _code(wdtype) if wdtype is not None else 0, float(eps), _ptr(out), _ptr(rows),
+                                      n_out, width, _stream()))
+    return out
+
+
+def rms_norm_cols(x: torch.Tensor, col0: int, n: int, weight: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """RMS norm of the columns col0 .. col0 + n of float32 rows -> [T, n] in out_dtype."""
+    _need_cuda(x, weight)
+    _rows2d("x", x)
+    if x.dtype != torch.float32 or col0 < 0 or n <= 0 or col0 + n > x.shape[1]:
+        raise ValueError(f"rms_norm_cols takes float32 rows and a run of columns inside them, got {x.dtype} {tuple(x.shape)} [{col0}, {col0 + n})")
+    if weight is not None and (weight.shape != (n,) or not weight.is_contiguous()):
+        raise ValueError(f"the norm weight must be a contiguous [{n}] tensor")
+    out = torch.empty(x.shape[0], n, dtype=out_dtype, device=x.device)
+    check(load().fmsamd_rms_norm_cols(x.data_ptr(), x.stride(0), col0, n, _ptr(weight), _code(weight.dtype) if weight is not None else 0,
+                                      float(eps), out.data_ptr(), _code(out_dtype), out.stride(0), x.shape[0], _stream()))
+    return out
+
+
+def activation(x: torch.Tensor, kind: str) -> torch.Tensor:
+    """act(x), elementwise, for the activations of ACTIVATIONS."""
+    _need_cuda(x)
+    if not x.is_contiguous():
+        raise ValueError("activation takes a contiguous tensor")
+    out = torch.empty_like(x)
+    check(load().fmsamd_activate(x.data_ptr(), out.data_ptr(), _code(x.dtype), x.numel(), ACTIVATIONS[kind], _stream()))
+    return out
+
+
+def clamped_gated_act(gu: torch.Tensor, limit: float, alpha: float, shift: float) -> torch.Tensor:
+    """[T, 2*hidden] (gate first) -> g' * sigmoid(alpha * g') * (u' + shift) with g' = min(g, limit) and
+    u' = clamp(u, -limit, limit)."""
+    _need_cuda(gu)
+    if gu.dim() != 2 or not gu.is_contiguous() or gu.shape[1] % 2:
+        raise ValueError("clamped_gated_act takes a contiguous [T, 2*hidden] tensor")
+    T, hidden = gu.shape[0], gu.shape[1] // 2
+    out = torch.empty(T, hidden, dtype=gu.dtype, device=gu.device)
+    for t0 in range(0, T, 65535):
+        n = min(65535, T - t0)
+        check(load().fmsamd_clamped_gated_act(gu[t0:].data_ptr(), out[t0:].data_ptr(), _code(gu.dtype), n, hidden, float(limit),
+                                              float(alpha), float(shift), _stream()))
+    return out
+
+
+# --------------------------------------------------------------------------
+# attention over a latent cache
+# --------------------------------------------------------------------------
+def _check_latent_cache(cache: torch.Tensor, width: int, dtype: torch.dtype) -> None:
+    if cache.dim() != 4 or tuple(cache.shape[1:]) != (1, PAGE_TOKENS, width) or not cache.is_contiguous() or cache.dtype != dtype:
+        raise ValueError(f"the latent cache must be contiguous {dtype} [pages, 1, {PAGE_TOKENS}, {width}], got {cache.dtype} {tuple(cache.shape)}")
+
+
+def _check_tables(cos, sin, rot: int) -> int:
+    if rot == 0:
+        return 0
+    if cos is None or sin is None or cos.dtype != torch.float32 or cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] * 2 != rot:
+        raise ValueError("cos/sin tables must be float32 [max_pos, rot/2]")
+    if not (cos.is_contiguous() and sin.is_contiguous()):
+        raise ValueError("cos/sin tables must be contiguous")
+    return cos.shape[0]
+
+
+def latent_kv_write(down: torch.Tensor, col0: int, rank: int, rot: int, norm_weight: Optional[torch.Tensor], eps: float,
+                    positions, seq_of_token, block_table, cos, sin, cache: torch.Tensor) -> None:
+    """From float32 rows whose columns col0 .. col0 + rank + rot hold a token's latent and shared key part: the
+    RMS-normed latent and the rotated key part go into the token's row of the latent cache."""
+    _need_cuda(down, norm_weight, positions, seq_of_token, block_table, cos, sin, cache)
+    _rows2d("down", down)
+    T = down.shape[0]
+    if down.dtype != torch.float32 or col0 < 0 or col0 + rank + rot > down.shape[1]:
+        raise ValueError("latent_kv_write takes float32 rows that hold the latent and the shared key part")
+    if norm_weight is not None and (norm_weight.shape != (rank,) or not norm_weight.is_contiguous()):
+        raise ValueError(f"the latent's norm weight must be a contiguous [{rank}] tensor")
+    _check_batch_index(positions, seq_of_token, block_table, T)
+    _check_latent_cache(cache, rank + rot, cache.dtype)
+    max_pos = _check_tables(cos, sin, rot)
+    check(load().fmsamd_latent_kv_write(down.data_ptr(), down.stride(0), col0, rank, rot, _ptr(norm_weight),
+                                        _code(norm_weight.dtype) if norm_weight is not None else 0, float(eps), positions.data_ptr(),
+                                        seq_of_token.data_ptr(), block_table.data_ptr(), block_table.stride(0), _ptr(cos), _ptr(sin),
+                                        max_pos, cache.data_ptr(), _code(cache.dtype), T, _stream()))
+
+
+def latent_q_rotate(q: torch.Tensor, qa: torch.Tensor, nheads: int, dim: int, rot: int, rank: int, positions, cos, sin) -> None:
+    """The rotated part of every head's query, q[t, h, dim:], rotated into qa[t, h, rank:]."""
+    _need_cuda(q, qa, positions, cos, sin)
+    _rows2d("q", q)
+    _rows2d("qa", qa)
+    if q.dtype != qa.dtype or q.shape[0] != qa.shape[0] or q.shape[1] != nheads * (dim + rot) or qa.shape[1] != nheads * (rank + rot):
+        raise ValueError("latent_q_rotate: q is [T, H*(dim+rot)] and qa [T, H*(rank+rot)] of one type")
+    _need_i32("positions", positions)
+    if positions.numel() < q.shape[0]:
+        raise ValueError("a position per token is needed")
+    max_pos = _check_tables(cos, sin, rot)
+    check(load().fmsamd_latent_q_rotate(q.data_ptr(), q.stride(0), _code(q.dtype), nheads, dim, rot, qa.data_ptr(), qa.stride(0), rank,
+                                        positions.data_ptr(), _ptr(cos), _ptr(sin), max_pos, q.shape[0], _stream()))
+
+
+def headwise_linear(x: torch.Tensor, x_head_stride: int, weight: torch.Tensor, y: torch.Tensor, y_head_stride: int,
+                    gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y[t, h*ys : h*ys + N] = weight[h] @ x[t, h*xs : h*xs + K] for weight [H, N, K]; with `gate` (float32 logits
+    [T, >= H], row-major) the result is multiplied by sigmoid(gate[t, h]).  x and y are 2-D rows."""
+    _need_cuda(x, weight, y, gate)
+    _rows2d("x", x)
+    _rows2d("y", y)
+    if weight.dim() != 3 or not weight.is_contiguous() or weight.dtype != x.dtype or y.dtype != x.dtype:
+        raise ValueError("headwise_linear takes a contiguous weight [H, N, K] of the type of x and y")
+    H, N, K = weight.shape
+    T = x.shape[0]
+    if y.shape[0] != T or x.shape[1] < (H - 1) * x_head_stride + K or y.shape[1] < (H - 1) * y_head_stride + N:
+        raise ValueError("headwise_linear: the rows of x or y are too short for the heads")
+    if gate is not None and (gate.dtype != torch.float32 or gate.dim() != 2 or gate.stride(1) != 1 or gate.shape[0] != T or gate.shape[1] < H):
+        raise ValueError("the gate is float32 [T, >= H] with contiguous rows")
+    for t0 in range(0, T, 65535 * 16):
+        n = min(65535 * 16, T - t0)
+        check(load().fmsamd_headwise_linear(x[t0:].data_ptr(), x.stride(0), x_head_stride, weight.data_ptr(), y[t0:].data_ptr(), y.stride(0),
+                                            y_head_stride, _ptr(gate[t0:]) if gate is not None else None, gate.stride(0) if gate is not None else 0,
+                                            _code(x.dtype), n, H, N, K, _stream()))
+    return y
+
+
+def latent_attention(qa: torch.Tensor, positions, seq_of_token, block_table, cache: torch.Tensor, sink: Optional[torch.Tensor],
+                     nheads: int, rank: int, rot: int, scale: float, window: int = 0, *, decode: bool = False,
+                     max_context: int = 0, force_generic: bool = False) -> torch.Tensor:
+    """Causal attention of every token over the latent cache of its sequence: qa [T, H*(rank+rot)] holds every head's
+    query in the space of the cache rows; returns sum_j p_j latent_j per head, [T, H*rank].  sink: float32 [H] or None."""
+    _need_cuda(qa, positions, seq_of_token, block_table, cache, sink)
+    _rows2d("qa", qa)
+    T = qa.shape[0]
+    if qa.shape[1] != nheads * (rank + rot):
+        raise ValueError(f"qa has {qa.shape[1]} columns, expected {nheads * (rank + rot)}")
+    _check_batch_index(positions, seq_of_token, block_table, T)
+    _check_latent_cache(cache, rank + rot, qa.dtype)
+    if sink is not None and (sink.dtype != torch.float32 or tuple(sink.shape) != (nheads,) or not sink.is_contiguous()):
+        raise ValueError(f"the sink is a contiguous float32 [{nheads}] tensor")
+    out = torch.empty(T, nheads * rank, dtype=qa.dtype, device=qa.device)
+    lib = load()
+    for t0 in range(0, T, 65535):
+        n = min(65535, T - t0)
+        check(lib.fmsamd_latent_attn_generic(qa[t0:].data_ptr(), qa.stride(0), out[t0:].data_ptr(), out.stride(0), _code(qa.dtype),
+                                             positions[t0:].data_ptr(), seq_of_token[t0:].data_ptr(), block_table.data_ptr(),
+                                             block_table.stride(0), cache.data_ptr(), _ptr(sink), n, nheads, rank, rot, float(scale),
+                                             int(window), _stream()))
+    return out
+
+
+# --------------------------------------------------------------------------
+# experts
+# --------------------------------------------------------------------------
+def moe_route(logits: torch.Tensor, n_experts: int, top: int):
+    """float32 logits [T, >= n_experts] -> (int32 ids [T, top], float32 weights [T, top]): the `top` largest logits of
+    every token among the first n_experts columns, and the softmax over those alone."""
+    _need_cuda(logits)
+    _rows2d("logits", logits)
+    if logits.dtype != torch.float32 or logits.shape[1] < n_experts:
+        raise ValueError("router logits are float32 [T, >= experts]")
+    T = logits.shape[0]
+    ids = torch.empty(T, top, dtype=torch.int32, device=logits.device)
+    weights = torch.empty(T, top, dtype=torch.float32, device=logits.device)
+    check(load().fmsamd_moe_route(logits.data_ptr(), logits.stride(0), T, n_experts, top, ids.data_ptr(), weights.data_ptr(), _stream()))
+    return ids, weights
+
+
+def moe_experts(x: torch.Tensor, ids: torch.Tensor, gate_w: torch.Tensor, up_w: torch.Tensor, down_w: torch.Tensor,
+                limit: float, alpha: float, shift: float) -> torch.Tensor:
+    """Every (token, choice) pair through its expert: float32 [T * top, width], row t * top + j the output of expert
+    ids[t, j] for token t.  gate_w, up_w [E, ff, width], down_w [E, width, ff]."""
+    _need_cuda(x, ids, gate_w, up_w, down_w)
+    _rows2d("x", x)
+    _need_i32("ids", ids)
+    T, top = ids.shape
+    E, ff, width = gate_w.shape
+    if x.shape != (T, width) or tuple(up_w.shape) != (E, ff, width) or tuple(down_w.shape) != (E, width, ff):
+        raise ValueError("moe_experts: x [T, width], gate and up [E, ff, width], down [E, width, ff]")
+    for w in (gate_w, up_w, down_w):
+        if w.dtype != x.dtype or not w.is_contiguous():
+            raise TypeError("the experts' weights are contiguous and of the type of x")
+    lib = load()
+    n_pairs = T * top
+    max_tiles = lib.fmsamd_moe_max_tiles(n_pairs, E)
+    order = torch.empty(n_pairs, dtype=torch.int32, device=x.device)
+    tiles = torch.empty(max_tiles, 3, dtype=torch.int32, device=x.device)
+    check(lib.fmsamd_moe_group(ids.data_ptr(), n_pairs, E, order.data_ptr(), tiles.data_ptr(), max_tiles, _stream()))
+    hidden = torch.empty(n_pairs, ff, dtype=x.dtype, device=x.device)
+    y = torch.empty(n_pairs, width, dtype=torch.float32, device=x.device)
+    code = _code(x.dtype)
+    check(lib.fmsamd_moe_experts(0, x.data_ptr(), x.stride(0), gate_w.data_ptr(), up_w.data_ptr(), hidden.data_ptr(), code,
+                                 order.data_ptr(), tiles.data_ptr(), max_tiles, top, ff, width, float(limit), float(alpha), float(shift), _stream()))
+    check(lib.fmsamd_moe_experts(1, hidden.data_ptr(), hidden.stride(0), down_w.data_ptr(), None, y.data_ptr(), code,
+                                 order.data_ptr(), tiles.data_ptr(), max_tiles, top, width, ff, float(limit), float(alpha), float(shift), _stream()))
+    return y
+
+
+def moe_combine(y: torch.Tensor, weights: torch.Tensor, shared: Optional[torch.Tensor], shared_gate: Optional[torch.Tensor],
+                out_dtype: torch.dtype) -> torch.Tensor:
+    """out[t] = sum_j weights[t, j] * y[t * top + j] (+ sigmoid(shared_gate[t]) * shared[t]) in out_dtype.
+    shared_gate: a float32 column view [T] (any row stride) of logits, or None for an ungated shared output."""
+    _need_cuda(y, weights, shared, shared_gate)
+    T, top = weights.shape
+    if y.dtype != torch.float32 or y.dim() != 2 or y.shape[0] != T * top or not y.is_contiguous() or not weights.is_contiguous() or weights.dtype != torch.float32:
+        raise ValueError("moe_combine: y is contiguous float32 [T * top, width], weights float32 [T, top]")
+    width = y.shape[1]
+    if shared is not None and (tuple(shared.shape) != (T, width) or shared.dtype != out_dtype or not shared.is_contiguous()):
+        raise ValueError("the shared expert's output is contiguous [T, width] of the output type")
+    ldg = 0
+    if shared_gate is not None:
+        if shared is None or shared_gate.dtype != torch.float32 or shared_gate.dim() != 1 or shared_gate.shape[0] != T:
+            raise ValueError("the shared gate is a float32 [T] view and needs a shared output")
+        ldg = shared_gate.stride(0)
+    out = torch.empty(T, width, dtype=out_dtype, device=y.device)
+    check(load().fmsamd_moe_combine(y.data_ptr(), weights.data_ptr(), top, _ptr(shared), _ptr(shared_gate), ldg, out.data_ptr(),
+                                    _code(out_dtype), T, width, _stream()))
+    return out
 
 
 # --------------------------------------------------------------------------

@@ -30,6 +30,7 @@ class ResidualStream:
     def __init__(self, resid: torch.Tensor):
         self.resid = resid
         self.pending: Optional[torch.Tensor] = None
+        self.pending_norm: Optional[Part] = None  # the norm that the pending branch passes before it is added
         self.prepared: Optional[tuple] = None  # (norm, NormedRows) of the stream as it is now
 
     def normed(self, norm: Part, act_dtype: torch.dtype, deferred_ok: bool = False, rows: Optional[torch.Tensor] = None):
@@ -38,12 +39,22 @@ class ResidualStream:
         if prepared is not None and prepared[0] is norm and deferred_ok and rows is None and self.fuse_products:
             return prepared[1]
         pending, self.pending = self.pending, None
+        pending_norm, self.pending_norm = self.pending_norm, None
+        if pending_norm is not None:
+            return norm.add_norm(self.resid, pending, act_dtype, rows, branch_norm=pending_norm)
         return norm.add_norm(self.resid, pending, act_dtype, rows)
 
-    def add_branch(self, out, next_norm: Optional[Part] = None) -> None:
-        """Takes a branch's output: a tensor (added when the stream is next read) or a BranchOutput."""
+    def add_branch(self, out, next_norm: Optional[Part] = None, post_norm: Optional[Part] = None) -> None:
+        """Takes a branch's output: a tensor (added when the stream is next read) or a BranchOutput.  post_norm: the
+        branch joins the stream through that norm (the norm that reads the stream next applies both)."""
         if self.pending is not None:
             raise RuntimeError("a branch output is still to be added: read the stream through a norm between two branches")
+        if post_norm is not None:
+            # the branch's norm needs the whole row of the branch: its last product cannot add into the stream
+            self.pending = out.value() if isinstance(out, BranchOutput) else out
+            self.pending_norm = post_norm
+            self.prepared = None
+            return
         if isinstance(out, BranchOutput):
             lin = out.linear
             if (self.fuse_products and next_norm is not None and getattr(next_norm, "deferrable", lambda: False)()
@@ -85,4 +96,35 @@ class PreNormBlock(Part):
         stream.add_branch(branch(h), next_norm)
 
 
+class SandwichNormBlock(Part):
+    """A block whose branches are normed on both sides: h = x + norm1b(mixer(norm1(x))); y = h + norm2b(ff(norm2(h))).
+    The feed-forward may be absent (None): the block is then its mixer branch alone.  The norm behind a branch, the
+    residual sum and the norm in front of the next branch are one kernel."""
+
+    norm_arguments = ("norm1", "norm1b", "norm2", "norm2b")
+
+    def __init__(self, mixer: Part, feed_forward: Optional[Part], norm1: Part, norm1b: Part, norm2: Part, norm2b: Part,
+                 names=("norm1", "mix", "norm1b", "norm2", "mlp", "norm2b")):
+        super().__init__()
+        self.norm1 = self.add_child(names[0], norm1)
+        self.mixer = self.add_child(names[1], mixer)
+        self.norm1b = self.add_child(names[2], norm1b)
+        self.feed_forward = feed_forward
+        if feed_forward is not None:
+            self.norm2 = self.add_child(names[3], norm2)
+            self.add_child(names[4], feed_forward)
+            self.norm2b = self.add_child(names[5], norm2b)
+
+    def first_norm(self) -> Part:
+        return self.norm1
+
+    def forward(self, stream: ResidualStream, batch, cache, act_dtype: torch.dtype, next_norm: Optional[Part] = None) -> None:
+        h = stream.normed(self.norm1, act_dtype)
+        stream.add_branch(self.mixer.forward(h, batch, cache), post_norm=self.norm1b)
+        if self.feed_forward is not None:
+            h = stream.normed(self.norm2, act_dtype)
+            stream.add_branch(self.feed_forward.forward(h), post_norm=self.norm2b)
+
+
 register_part("block", "pre_norm", PreNormBlock)
+register_part("block", "sandwich_norm", SandwichNormBlock)

@@ -13,15 +13,15 @@ from .base import Part, register_part
 
 
 class TokenEmbedding(Part):
-    def __init__(self, vocab: int, width: int):
+    def __init__(self, vocab: int, width: int, scale: float = 1.0):
         super().__init__()
-        self.vocab, self.width = vocab, width
+        self.vocab, self.width, self.scale = vocab, width, float(scale)  # scale: a constant factor on every row
         self.declare("weight", (vocab, width))
 
     def forward(self, token_ids: torch.Tensor, batch=None) -> torch.Tensor:
         """int32 ids [T] -> the float32 residual stream [T, width].  `batch` is the step (positions, sequence of
         every token): an embedding that adds a learned vector per position reads it, this one does not."""
-        return ops.embed(token_ids, self.w["weight"])
+        return ops.embed(token_ids, self.w["weight"], self.scale)
 
 
 class LinearHead(Part):

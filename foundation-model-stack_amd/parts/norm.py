@@ -38,8 +38,16 @@ class ParameterizedNorm(Part):
         branch: Optional[torch.Tensor],
         out_dtype: torch.dtype,
         rows: Optional[torch.Tensor] = None,
+        branch_norm: Optional["ParameterizedNorm"] = None,
     ) -> torch.Tensor:
-        """resid += branch (float32, in place); returns norm(resid) in out_dtype (only `rows` if given)."""
+        """resid += branch (float32, in place); returns norm(resid) in out_dtype (only `rows` if given).
+        branch_norm: the branch goes through that norm first (a block that norms its branches before they join the
+        stream); both norms and the sum are then one kernel."""
+        if branch_norm is not None and branch is not None:
+            if not (self.deferrable() and branch_norm.deferrable()):
+                raise NotImplementedError("a normed branch is added by RMS norms without mean and shift only")
+            return ops.norm_add_norm(resid, branch, branch_norm.w.get("weight"), branch_norm.eps, self.w.get("weight"), self.eps,
+                                     out_dtype, rows)
         return ops.add_norm(resid, branch, self.w.get("weight"), self.w.get("bias"), self.eps, out_dtype, rows, self.use_mean)
 
     def deferrable(self) -> bool:

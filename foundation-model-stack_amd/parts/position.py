@@ -34,7 +34,7 @@ def ntk_alpha(length: int, original_length: int) -> int:
     return 1 << (ratio - 1).bit_length()
 
 
-def rope_frequencies(dim: int, theta: float, scaling: Optional[dict] = None, alpha: int = 1) -> torch.Tensor:
+def rope_frequencies(dim: int, theta: float, scaling: Optional[dict] = None, alpha: int = 1, exact: bool = False) -> torch.Tensor:
     """Float32 frequencies f_i, i < dim/2.
 
     regular: fms/modules/positions.py:124-132.  llama3: fms/modules/positions.py:171-196.
@@ -44,7 +44,11 @@ def rope_frequencies(dim: int, theta: float, scaling: Optional[dict] = None, alp
     kind = scaling.get("rope_type", "regular")
     if kind == "ntk":
         theta = theta * alpha ** (dim / (dim - 2))
-    freqs = 1.0 / (theta ** (torch.arange(0, dim, 2)[: dim // 2].float() / dim))
+    if exact:
+        # theta^(-2i/dim) formed in float64 and rounded once, for models that define the frequencies as real numbers
+        freqs = torch.tensor([float(theta) ** (-2.0 * i / dim) for i in range(dim // 2)], dtype=torch.float64).to(torch.float32)
+    else:
+        freqs = 1.0 / (theta ** (torch.arange(0, dim, 2)[: dim // 2].float() / dim))
     if kind in ("regular", "ntk"):
         return freqs
     if kind == "llama3":
@@ -89,8 +93,9 @@ class RotaryEncoding(PositionEncoding):
     the encoding is the regular one (tests/modules/test_positions.py:216-241)."""
 
     def __init__(self, dim: int, theta: float = 10_000.0, max_seq_len: int = 2048, scaling: Optional[dict] = None,
-                 partial_rope: float = 1.0, max_positions: Optional[int] = None):
+                 partial_rope: float = 1.0, max_positions: Optional[int] = None, exact_frequencies: bool = False):
         super().__init__()
+        self.exact_frequencies = bool(exact_frequencies)
         self.head_dim = dim
         self.rot_dim = int(partial_rope * dim)
         if self.rot_dim % 2 or self.rot_dim <= 0 or self.rot_dim > dim:
@@ -100,7 +105,7 @@ class RotaryEncoding(PositionEncoding):
         self.max_positions = int(max_positions) if (max_positions and self.stretches) else self.max_seq_len
         if self.stretches and self.rot_dim <= 2:
             raise ValueError("ntk scaling needs a rotary size above 2")
-        self.freqs = rope_frequencies(self.rot_dim, self.theta, self.scaling)
+        self.freqs = rope_frequencies(self.rot_dim, self.theta, self.scaling, exact=self.exact_frequencies)
         self.cos: Optional[torch.Tensor] = None
         self.sin: Optional[torch.Tensor] = None
         self.tables = {}  # alpha -> (cos, sin); alpha 1 only unless the encoding stretches
@@ -114,7 +119,7 @@ class RotaryEncoding(PositionEncoding):
         alpha = 1
         while True:
             length = min(self.max_seq_len * alpha, self.max_positions)
-            freqs = rope_frequencies(self.rot_dim, self.theta, self.scaling, alpha)
+            freqs = rope_frequencies(self.rot_dim, self.theta, self.scaling, alpha, exact=self.exact_frequencies)
             self.tables[alpha] = ops.rope_table(freqs.to(device), length)
             if self.max_seq_len * alpha >= self.max_positions:
                 break

@@ -22,7 +22,7 @@ class PartSpec:
 @dataclasses.dataclass
 class LayerSpec:
     mixer: PartSpec
-    feed_forward: PartSpec
+    feed_forward: Optional[PartSpec]  # None: the layer has none (its block must take that)
     norm: Optional[PartSpec] = None  # the spec of every norm the block asks for ...
     block: PartSpec = dataclasses.field(default_factory=lambda: PartSpec("pre_norm"))
     position: Optional[str] = None  # key into ModelSpec.positions, handed to the mixer

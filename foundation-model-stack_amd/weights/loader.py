@@ -48,7 +48,7 @@ def kept_dtype(stored: torch.dtype, kind: str, model_dtype: torch.dtype, forced:
     return model_dtype
 
 
-_LAYER = re.compile(r"(^|\.)(\d+)\.")
+_LAYER = re.compile(r"(^|\.)[A-Za-z]?(\d+)\.")  # "layers.3." and "l3." alike
 
 
 def _layer_groups(names: List[str]) -> List[List[str]]:
