@@ -37,6 +37,7 @@ class KVNeed:
     # False: one tensor of rows [page][kv head][token][head_dim] and no value tensor (a mixer whose values are a part
     # or a function of what it keeps as keys, like attention over a latent)
     values: bool = True
+    value_dim: int = 0  # size of a value if it is not head_dim (0: head_dim)
 
 
 @dataclasses.dataclass(frozen=True)
@@ -64,10 +65,11 @@ class KVGroup:
         # zero-filled: the attention kernels multiply masked-out positions by zero
         self.keys = torch.zeros(len(self.entries), n, K, PAGE_TOKENS, D, dtype=dtype, device=device)
         if self.need.values:
-            self.values = torch.zeros(len(self.entries), n, K, D, PAGE_TOKENS, dtype=dtype, device=device)
+            self.values = torch.zeros(len(self.entries), n, K, self.need.value_dim or D, PAGE_TOKENS, dtype=dtype, device=device)
 
     def bytes_per_token(self, itemsize: int) -> int:
-        return (2 if self.need.values else 1) * len(self.entries) * self.need.kv_heads * self.need.head_dim * itemsize
+        per_head = self.need.head_dim + ((self.need.value_dim or self.need.head_dim) if self.need.values else 0)
+        return len(self.entries) * self.need.kv_heads * per_head * itemsize
 
 
 class SequenceCache:

@@ -183,12 +183,13 @@ int fmsamd_clamped_gated_act(const void* gu, void* out, int dtype, int n_tokens,
 
 // ---- attention over a latent cache (latent_attention.hip) ---------------------------------------------------------
 // The cache holds one row [rank + rot] per token: pages [page][token in page][rank + rot].
+// vt_cache (or null): the latent once more, transposed, pages [page][rank][token in page], for the MFMA kernel.
 // down: float32 rows whose columns col0 .. col0 + rank + rot are the latent before its norm and the shared key part
 // before its rotation; the normed latent and the rotated part are written into the token's page.
 int fmsamd_latent_kv_write(const float* down, long ld, int col0, int rank, int rot, const void* norm_weight,
                            int weight_dtype, float eps, const int* positions, const int* seq_of_token,
                            const int* block_table, int table_stride, const float* cos_t, const float* sin_t, int max_pos,
-                           void* cache, int cache_dtype, int n_tokens, hipStream_t stream);
+                           void* cache, void* vt_cache, int cache_dtype, int n_tokens, hipStream_t stream);
 // qa[t, h, rank : rank + rot] = rotate(q[t, h, dim : dim + rot]); q rows hold nheads x (dim + rot), qa rows nheads x (rank + rot)
 int fmsamd_latent_q_rotate(const void* q, long ldq, int dtype, int nheads, int dim, int rot, void* qa, long ldqa, int rank,
                            const int* positions, const float* cos_t, const float* sin_t, int max_pos, int n_tokens,
@@ -203,6 +204,16 @@ int fmsamd_latent_attn_generic(const void* qa, long ldq, void* out, long ldo, in
                                const int* seq_of_token, const int* block_table, int table_stride, const void* cache,
                                const float* sink, int n_tokens, int nheads, int rank, int rot, float scale, int window,
                                hipStream_t stream);
+
+// The same attention for bfloat16 on the matrix cores (sizes: fmsamd_latent_attn_mfma_fits).  n_splits 0: prompts;
+// n_splits >= 1: single tokens, every (token, 16 heads) dealt over n_splits blocks of four waves, partial results in
+// a workspace of fmsamd_latent_attn_workspace(...) bytes, merged by a second kernel.
+long fmsamd_latent_attn_workspace(int n_tokens, int nheads, int rank, int n_splits);
+int fmsamd_latent_attn_mfma_fits(int rank, int rot);
+int fmsamd_latent_attn_mfma(const void* qa, long ldq, void* out, long ldo, void* workspace, long workspace_bytes,
+                            const int* positions, const int* seq_of_token, const int* block_table, int table_stride,
+                            const void* cache, const void* vt_cache, const float* sink, int n_tokens, int nheads, int rank,
+                            int rot, float scale, int window, int n_splits, hipStream_t stream);
 
 // ---- experts (experts.hip) -----------------------------------------------------------------------------------------
 int fmsamd_moe_route(const float* logits, long ld, int n_tokens, int n_experts, int top, int* ids, float* weights,

@@ -13,9 +13,10 @@
 //   latent_q_rotate:      the rotated part of every head's query into its place behind the latent part
 //   headwise_linear:      y[t, h, :] = W_h x[t, h, :] (optionally times sigmoid(gate[t, h])), FMA or MFMA
 //   latent_attn_generic:  float32 arithmetic on any storage type; one block per (head, token)
-//   latent_attn_mfma:     bfloat16, a block per 16 (token, head) rows ... see below
+//   latent_attn_mfma:     bfloat16, MFMA 16x16x32; a wave owns 16 heads of one token (+ merge of partial results)
 //
-// Cache layout: rows [page][token in page][R + P].
+// Cache layout: rows [page][token in page][R + P]; for the MFMA kernel also the latent transposed, [page][R][token in
+// page], so that both products read their contraction index contiguously, straight from global memory.
 #include "common.h"
 #include "fmsamd.h"
 #include "tile_product.h"
@@ -28,7 +29,7 @@ __global__ void __launch_bounds__(256)
     latent_kv_write_kernel(const float* __restrict__ down, long ld, int col0, int rank, int rot, const void* __restrict__ w,
                            int w_dtype, float eps, const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                            const int* __restrict__ block_table, int table_stride, const float* __restrict__ cos_t,
-                           const float* __restrict__ sin_t, CT* __restrict__ cache) {
+                           const float* __restrict__ sin_t, CT* __restrict__ cache, CT* __restrict__ vt_cache) {
   __shared__ float scratch[17];
   const int t = blockIdx.x;
   const int seq = seq_of_token[t];
@@ -43,7 +44,11 @@ __global__ void __launch_bounds__(256)
   const float rs = rsqrtf(block_sum(sq, scratch) / (float)rank + eps);
   for (int i = threadIdx.x; i < rank; i += blockDim.x) {
     const float wi = w == nullptr ? 1.f : (w_dtype == FMS_F32 ? ((const float*)w)[i] : (float)((const bf16*)w)[i]);
-    row[i] = from_f32<CT>(x[i] * rs * wi);
+    const CT c = from_f32<CT>(x[i] * rs * wi);
+    row[i] = c;
+    // the latent once more with the tokens of a page side by side, [page][rank][token]: the layout from which the
+    // second product of the MFMA kernel loads its operand without a transposition
+    if (vt_cache) vt_cache[((size_t)page * rank + i) * PAGE_TOKENS + pos % PAGE_TOKENS] = c;
   }
   const int half = rot / 2;
   for (int i = threadIdx.x; i < half; i += blockDim.x) {
@@ -57,7 +62,8 @@ __global__ void __launch_bounds__(256)
 extern "C" int fmsamd_latent_kv_write(const float* down, long ld, int col0, int rank, int rot, const void* norm_weight,
                                       int weight_dtype, float eps, const int* positions, const int* seq_of_token,
                                       const int* block_table, int table_stride, const float* cos_t, const float* sin_t,
-                                      int max_pos, void* cache, int cache_dtype, int n_tokens, hipStream_t stream) {
+                                      int max_pos, void* cache, void* vt_cache, int cache_dtype, int n_tokens,
+                                      hipStream_t stream) {
   if (n_tokens == 0) return 0;
   FMS_REQUIRE(n_tokens > 0 && rank > 0 && rot >= 0 && rot % 2 == 0 && col0 >= 0 && ld >= col0 + rank + rot,
               "latent_kv_write: bad sizes T=%d rank=%d rot=%d col0=%d ld=%ld", n_tokens, rank, rot, col0, ld);
@@ -65,11 +71,11 @@ extern "C" int fmsamd_latent_kv_write(const float* down, long ld, int col0, int 
   if (cache_dtype == FMS_F32)
     latent_kv_write_kernel<float><<<n_tokens, 256, 0, stream>>>(down, ld, col0, rank, rot, norm_weight, weight_dtype, eps,
                                                                 positions, seq_of_token, block_table, table_stride, cos_t,
-                                                                sin_t, (float*)cache);
+                                                                sin_t, (float*)cache, (float*)vt_cache);
   else if (cache_dtype == FMS_BF16)
     latent_kv_write_kernel<bf16><<<n_tokens, 256, 0, stream>>>(down, ld, col0, rank, rot, norm_weight, weight_dtype, eps,
                                                                positions, seq_of_token, block_table, table_stride, cos_t,
-                                                               sin_t, (bf16*)cache);
+                                                               sin_t, (bf16*)cache, (bf16*)vt_cache);
   else
     FMS_REQUIRE(false, "latent_kv_write: unknown dtype %d", cache_dtype);
   FMS_LAUNCH_CHECK("latent_kv_write");
@@ -296,5 +302,220 @@ extern "C" int fmsamd_latent_attn_generic(const void* qa, long ldq, void* out, l
   else
     FMS_REQUIRE(false, "latent_attn_generic: unknown dtype %d", dtype);
   FMS_LAUNCH_CHECK("latent_attn_generic");
+  return 0;
+}
+
+
+// --------------------------------------------------------------------------
+// bfloat16 MFMA kernel.  A wave owns one token and 16 of its heads (the columns of its tiles) and walks over tiles of
+// 32 keys.  S^T = K Q^T (rows: keys, columns: heads) leaves the probabilities in the accumulator in the operand
+// layout of O^T = C^T P^T, so nothing goes through LDS.  The 32 keys of a tile are dealt to the two score tiles so
+// that a lane's eight probabilities are eight consecutive keys: tile a has the keys 8g + i, tile b the keys
+// 8g + 4 + i (g, i < 4).
+//
+// Two ways to share the work of a block's four waves:
+//   * prompts: each wave another (token, head group); every wave walks all keys of its token (the waves of a block
+//     read the same rows, which the caches serve);
+//   * single tokens: all waves of a block, and the blocks of several splits, share one (token, head group) and deal
+//     its key tiles out in turn; every part leaves (maximum, sum, unnormalised result) in a workspace and a second
+//     kernel merges them.
+// The sink starts the maximum of every part and is counted in the sum of part 0 only.
+// --------------------------------------------------------------------------
+#define LAT_EMPTY -1e30f
+
+template <int RT, int WC>
+__global__ void __launch_bounds__(256)
+    latent_attn_mfma_kernel(const bf16* __restrict__ qa, long ldq, bf16* __restrict__ out, long ldo, float* __restrict__ ws,
+                            const int* __restrict__ positions, const int* __restrict__ seq_of_token,
+                            const int* __restrict__ block_table, int table_stride, const bf16* __restrict__ cache,
+                            const bf16* __restrict__ vt_cache, const float* __restrict__ sink, int n_tokens, int nheads,
+                            int rank, int width, float scale, int window, int tiles_per_token, int n_parts) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  int tile, part;
+  if (n_parts == 1) {
+    tile = blockIdx.x * 4 + wave;
+    part = 0;
+  } else {
+    tile = blockIdx.x;
+    part = blockIdx.y * 4 + wave;
+  }
+  if (tile >= n_tokens * tiles_per_token) return;
+  const int t = tile / tiles_per_token;
+  const int head = (tile % tiles_per_token) * 16 + col;
+  const bool valid = head < nheads;
+  const int seq = uniform_load(seq_of_token + t);
+  if (seq < 0) {
+    if (n_parts == 1 && valid) {
+      for (int d = grp; d < rank; d += 4) out[(size_t)t * ldo + (size_t)head * rank + d] = (bf16)0.f;
+    }
+    return;
+  }
+  const int pos = uniform_load(positions + t);
+  const int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
+  const int* bt = block_table + (size_t)seq * table_stride;
+
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  bf16x8 qreg[WC];
+  {
+    const bf16* qrow = qa + (size_t)t * ldq + (size_t)(valid ? head : 0) * width;
+#pragma unroll
+    for (int c = 0; c < WC; ++c) {
+      const int k = c * 32 + grp * 8;
+      qreg[c] = (valid && k < width) ? *reinterpret_cast<const bf16x8*>(qrow + k) : zero8;
+    }
+  }
+  f32x4 acc[RT];
+#pragma unroll
+  for (int dt = 0; dt < RT; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = (sink && valid) ? sink[head] : LAT_EMPTY;
+  float l_run = (sink && valid && part == 0 && grp == 0) ? 1.f : 0.f;
+
+  const int key_a = 8 * (col >> 2) + (col & 3);  // the key of this lane's row in score tile a; tile b: + 4
+  for (int kt = lo / 32 + part; kt * 32 <= pos; kt += n_parts) {
+    const int base = kt * 32;
+    const size_t page = readable_page(uniform_load(bt + base / PAGE_TOKENS));
+    const int in_page = base % PAGE_TOKENS;
+    const bf16* ka = cache + (page * PAGE_TOKENS + in_page + key_a) * width + grp * 8;
+    const bf16* kb = ka + 4 * (size_t)width;
+    f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < WC; ++c) {
+      if (c * 32 < width) {
+        const bool in = c * 32 + grp * 8 < width;
+        const bf16x8 a = in ? *reinterpret_cast<const bf16x8*>(ka + c * 32) : zero8;
+        const bf16x8 b = in ? *reinterpret_cast<const bf16x8*>(kb + c * 32) : zero8;
+        sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qreg[c], sa, 0, 0, 0);
+        sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b, qreg[c], sb, 0, 0, 0);
+      }
+    }
+    // this lane's scores: keys base + 8 grp + i (sa) and base + 8 grp + 4 + i (sb) of column `col`
+    float s[8];
+    float top = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int ja = base + 8 * grp + i, jb = ja + 4;
+      s[i] = (ja >= lo && ja <= pos) ? sa[i] * scale : -INFINITY;
+      s[4 + i] = (jb >= lo && jb <= pos) ? sb[i] * scale : -INFINITY;
+      top = fmaxf(top, fmaxf(s[i], s[4 + i]));
+    }
+    top = fmaxf(top, __shfl_xor(top, 16, WAVE));
+    top = fmaxf(top, __shfl_xor(top, 32, WAVE));
+    const float m_new = fmaxf(m_run, top);
+    const float alpha = __expf(m_run - m_new);
+    float psum = 0.f;
+    bf16x8 pmat;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float p = __expf(s[i] - m_new);  // exp(-inf) = 0 for the keys that are not seen
+      psum += p;
+      pmat[i] = (bf16)p;
+    }
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+    const bf16* vt = vt_cache + (page * rank + col) * PAGE_TOKENS + in_page + grp * 8;
+#pragma unroll
+    for (int dt = 0; dt < RT; ++dt) {
+      if (dt * 16 < rank) {
+        const bf16x8 v = *reinterpret_cast<const bf16x8*>(vt + (size_t)dt * 16 * PAGE_TOKENS);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[dt][i] *= alpha;
+        acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pmat, acc[dt], 0, 0, 0);
+      }
+    }
+  }
+  l_run += __shfl_xor(l_run, 16, WAVE);
+  l_run += __shfl_xor(l_run, 32, WAVE);
+  if (!valid) return;
+  // acc[dt][i] is element d = dt * 16 + grp * 4 + i of column `col`
+  if (n_parts == 1) {
+    const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+    bf16* o = out + (size_t)t * ldo + (size_t)head * rank;
+#pragma unroll
+    for (int dt = 0; dt < RT; ++dt) {
+      if (dt * 16 < rank) {
+        bf16x4 r = {(bf16)(acc[dt][0] * inv), (bf16)(acc[dt][1] * inv), (bf16)(acc[dt][2] * inv), (bf16)(acc[dt][3] * inv)};
+        *reinterpret_cast<bf16x4*>(o + dt * 16 + grp * 4) = r;
+      }
+    }
+  } else {
+    float* w = ws + (((size_t)t * nheads + head) * n_parts + part) * (rank + 4);
+    if (grp == 0) w[0] = m_run, w[1] = l_run;
+#pragma unroll
+    for (int dt = 0; dt < RT; ++dt) {
+      if (dt * 16 < rank) *reinterpret_cast<f32x4*>(w + 4 + dt * 16 + grp * 4) = acc[dt];
+    }
+  }
+}
+
+// out[t, h, :] = sum_i acc_i exp(m_i - M) / sum_i l_i exp(m_i - M) over the parts i
+__global__ void __launch_bounds__(64)
+    latent_attn_merge_kernel(const float* __restrict__ ws, bf16* __restrict__ out, long ldo, const int* __restrict__ seq_of_token,
+                             int nheads, int rank, int n_parts) {
+  const int h = blockIdx.x, t = blockIdx.y;
+  bf16* o = out + (size_t)t * ldo + (size_t)h * rank;
+  if (seq_of_token[t] < 0) {
+    for (int d = threadIdx.x; d < rank; d += blockDim.x) o[d] = (bf16)0.f;
+    return;
+  }
+  const float* w = ws + ((size_t)t * nheads + h) * n_parts * (rank + 4);
+  float top = LAT_EMPTY;
+  for (int i = 0; i < n_parts; ++i) top = fmaxf(top, w[(size_t)i * (rank + 4)]);
+  float total = 0.f;
+  for (int i = 0; i < n_parts; ++i) total += w[(size_t)i * (rank + 4) + 1] * __expf(w[(size_t)i * (rank + 4)] - top);
+  const float inv = total > 0.f ? 1.f / total : 0.f;
+  for (int d = threadIdx.x; d < rank; d += blockDim.x) {
+    float v = 0.f;
+    for (int i = 0; i < n_parts; ++i) v = fmaf(w[(size_t)i * (rank + 4) + 4 + d], __expf(w[(size_t)i * (rank + 4)] - top), v);
+    o[d] = (bf16)(v * inv);
+  }
+}
+
+// bytes of the workspace for n_splits blocks of four parts each (0: one block per four tiles, no workspace)
+extern "C" long fmsamd_latent_attn_workspace(int n_tokens, int nheads, int rank, int n_splits) {
+  return n_splits <= 0 ? 0 : (long)n_tokens * nheads * n_splits * 4 * (rank + 4) * (long)sizeof(float);
+}
+
+// 1 if the MFMA kernel takes these sizes
+extern "C" int fmsamd_latent_attn_mfma_fits(int rank, int rot) {
+  return rank > 0 && rank % 16 == 0 && rot >= 0 && (rank + rot) % 8 == 0 && rank <= 512 && rank + rot <= 576;
+}
+
+// n_splits 0: prompts (a wave per tile, every wave all keys); n_splits >= 1: single tokens (n_splits blocks of four
+// waves deal a tile's keys out; workspace as fmsamd_latent_attn_workspace says)
+extern "C" int fmsamd_latent_attn_mfma(const void* qa, long ldq, void* out, long ldo, void* workspace, long workspace_bytes,
+                                       const int* positions, const int* seq_of_token, const int* block_table,
+                                       int table_stride, const void* cache, const void* vt_cache, const float* sink,
+                                       int n_tokens, int nheads, int rank, int rot, float scale, int window, int n_splits,
+                                       hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  const int width = rank + rot;
+  FMS_REQUIRE(n_tokens > 0 && nheads > 0 && fmsamd_latent_attn_mfma_fits(rank, rot), "latent_attn_mfma: sizes T=%d H=%d rank=%d rot=%d do not fit",
+              n_tokens, nheads, rank, rot);
+  FMS_REQUIRE(ldq >= (long)nheads * width && ldq % 8 == 0 && ldo >= (long)nheads * rank && ldo % 4 == 0 && ((uintptr_t)qa % 16) == 0,
+              "latent_attn_mfma: rows too short or not aligned");
+  FMS_REQUIRE(cache != nullptr && vt_cache != nullptr && window >= 0 && n_splits >= 0 && n_splits <= 16384, "latent_attn_mfma: bad arguments");
+  const int tiles_per_token = ceil_div(nheads, 16);
+  const long tiles = (long)n_tokens * tiles_per_token;
+  const int n_parts = n_splits == 0 ? 1 : n_splits * 4;
+  FMS_REQUIRE(n_splits == 0 || (workspace != nullptr && workspace_bytes >= fmsamd_latent_attn_workspace(n_tokens, nheads, rank, n_splits)),
+              "latent_attn_mfma: the workspace is too small");
+  const dim3 grid(n_splits == 0 ? ceil_div(tiles, 4) : (unsigned)tiles, n_splits == 0 ? 1 : n_splits);
+  FMS_REQUIRE(tiles <= 0x7fffffffL && grid.y <= 65535, "latent_attn_mfma: too many tiles for one launch");
+#define LAUNCH_LATENT(RT, WC)                                                                                                  \
+  latent_attn_mfma_kernel<RT, WC><<<grid, 256, 0, stream>>>((const bf16*)qa, ldq, (bf16*)out, ldo, (float*)workspace, positions, \
+                                                            seq_of_token, block_table, table_stride, (const bf16*)cache,       \
+                                                            (const bf16*)vt_cache, sink, n_tokens, nheads, rank, width, scale, \
+                                                            window, tiles_per_token, n_parts)
+  if (rank <= 128 && width <= 192) LAUNCH_LATENT(8, 6);
+  else if (rank <= 256 && width <= 320) LAUNCH_LATENT(16, 10);
+  else LAUNCH_LATENT(32, 18);
+#undef LAUNCH_LATENT
+  FMS_LAUNCH_CHECK("latent_attn_mfma");
+  if (n_parts > 1) {
+    latent_attn_merge_kernel<<<dim3(nheads, n_tokens), 64, 0, stream>>>((const float*)workspace, (bf16*)out, ldo, seq_of_token, nheads,
+                                                                         rank, n_parts);
+    FMS_LAUNCH_CHECK("latent_attn_merge");
+  }
   return 0;
 }

@@ -51,7 +51,8 @@ _SIGNATURES = {
     "fmsamd_rms_norm_cols": [P, L, I, I, P, I, F, P, I, L, I, P],
     "fmsamd_activate": [P, P, I, L, I, P],
     "fmsamd_clamped_gated_act": [P, P, I, I, I, F, F, F, P],
-    "fmsamd_latent_kv_write": [P, L, I, I, I, P, I, F, P, P, P, I, P, P, I, P, I, I, P],
+    "fmsamd_latent_kv_write": [P, L, I, I, I, P, I, F, P, P, P, I, P, P, I, P, P, I, I, P],
+    "fmsamd_latent_attn_mfma": [P, L, P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, F, I, I, P],
     "fmsamd_latent_q_rotate": [P, L, I, I, I, I, P, L, I, P, P, P, I, I, P],
     "fmsamd_headwise_linear": [P, L, L, P, P, L, L, P, L, I, I, I, I, I, P],
     "fmsamd_latent_attn_generic": [P, L, P, L, I, P, P, P, I, P, P, I, I, I, I, F, I, P],
@@ -98,6 +99,10 @@ def load(verbose: bool = True) -> ctypes.CDLL:
             fn.restype = c_int
         lib.fmsamd_attn_prefill_qblock.restype = c_int
         lib.fmsamd_attn_prefill_qblock.argtypes = [I, I, I, I]
+        lib.fmsamd_latent_attn_workspace.restype = c_long
+        lib.fmsamd_latent_attn_workspace.argtypes = [I, I, I, I]
+        lib.fmsamd_latent_attn_mfma_fits.restype = c_int
+        lib.fmsamd_latent_attn_mfma_fits.argtypes = [I, I]
         lib.fmsamd_moe_max_tiles.restype = c_int
         lib.fmsamd_moe_max_tiles.argtypes = [I, I]
         lib.fmsamd_argmax_workspace.restype = c_long

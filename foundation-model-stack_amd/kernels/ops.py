@@ -678,6 +678,24 @@ def _check_latent_cache(cache: torch.Tensor, width: int, dtype: torch.dtype) -> 
         raise ValueError(f"the latent cache must be contiguous {dtype} [pages, 1, {PAGE_TOKENS}, {width}], got {cache.dtype} {tuple(cache.shape)}")
 
 
+def _check_latent_values(vt_cache: Optional[torch.Tensor], cache: torch.Tensor, rank: int) -> None:
+    if vt_cache is not None and (vt_cache.dim() != 4 or tuple(vt_cache.shape) != (cache.shape[0], 1, rank, PAGE_TOKENS)
+                                 or not vt_cache.is_contiguous() or vt_cache.dtype != cache.dtype):
+        raise ValueError(f"the transposed latent cache must be contiguous {cache.dtype} [{cache.shape[0]}, 1, {rank}, {PAGE_TOKENS}]")
+
+
+def latent_attention_fits_mfma(rank: int, rot: int) -> bool:
+    """True if the matrix-core kernel of the latent attention takes these sizes (the library says)."""
+    return bool(load().fmsamd_latent_attn_mfma_fits(int(rank), int(rot)))
+
+
+def latent_attention_splits(n_tokens: int, nheads: int, max_context: int) -> int:
+    """How many blocks share one (token, 16 heads) of the decode step of the MFMA kernel: enough for a few hundred
+    blocks in all, and no block with fewer than four tiles of 32 keys (one for each of its waves)."""
+    tiles = n_tokens * -(-nheads // 16)
+    return max(1, min(-(-512 // tiles), -(-max_context // 32) // 4, 64))
+
+
 def _check_tables(cos, sin, rot: int) -> int:
     if rot == 0:
         return 0
@@ -689,10 +707,11 @@ def _check_tables(cos, sin, rot: int) -> int:
 
 
 def latent_kv_write(down: torch.Tensor, col0: int, rank: int, rot: int, norm_weight: Optional[torch.Tensor], eps: float,
-                    positions, seq_of_token, block_table, cos, sin, cache: torch.Tensor) -> None:
+                    positions, seq_of_token, block_table, cos, sin, cache: torch.Tensor, vt_cache: Optional[torch.Tensor] = None) -> None:
     """From float32 rows whose columns col0 .. col0 + rank + rot hold a token's latent and shared key part: the
-    RMS-normed latent and the rotated key part go into the token's row of the latent cache."""
-    _need_cuda(down, norm_weight, positions, seq_of_token, block_table, cos, sin, cache)
+    RMS-normed latent and the rotated key part go into the token's row of the latent cache; with vt_cache
+    [pages, 1, rank, 64] the latent also goes there, transposed."""
+    _need_cuda(down, norm_weight, positions, seq_of_token, block_table, cos, sin, cache, vt_cache)
     _rows2d("down", down)
     T = down.shape[0]
     if down.dtype != torch.float32 or col0 < 0 or col0 + rank + rot > down.shape[1]:
@@ -701,11 +720,12 @@ def latent_kv_write(down: torch.Tensor, col0: int, rank: int, rot: int, norm_wei
         raise ValueError(f"the latent's norm weight must be a contiguous [{rank}] tensor")
     _check_batch_index(positions, seq_of_token, block_table, T)
     _check_latent_cache(cache, rank + rot, cache.dtype)
+    _check_latent_values(vt_cache, cache, rank)
     max_pos = _check_tables(cos, sin, rot)
     check(load().fmsamd_latent_kv_write(down.data_ptr(), down.stride(0), col0, rank, rot, _ptr(norm_weight),
                                         _code(norm_weight.dtype) if norm_weight is not None else 0, float(eps), positions.data_ptr(),
                                         seq_of_token.data_ptr(), block_table.data_ptr(), block_table.stride(0), _ptr(cos), _ptr(sin),
-                                        max_pos, cache.data_ptr(), _code(cache.dtype), T, _stream()))
+                                        max_pos, cache.data_ptr(), _ptr(vt_cache), _code(cache.dtype), T, _stream()))
 
 
 def latent_q_rotate(q: torch.Tensor, qa: torch.Tensor, nheads: int, dim: int, rot: int, rank: int, positions, cos, sin) -> None:
@@ -748,10 +768,14 @@ def headwise_linear(x: torch.Tensor, x_head_stride: int, weight: torch.Tensor, y
 
 def latent_attention(qa: torch.Tensor, positions, seq_of_token, block_table, cache: torch.Tensor, sink: Optional[torch.Tensor],
                      nheads: int, rank: int, rot: int, scale: float, window: int = 0, *, decode: bool = False,
-                     max_context: int = 0, force_generic: bool = False) -> torch.Tensor:
+                     max_context: int = 0, force_generic: bool = False, vt_cache: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal attention of every token over the latent cache of its sequence: qa [T, H*(rank+rot)] holds every head's
-    query in the space of the cache rows; returns sum_j p_j latent_j per head, [T, H*rank].  sink: float32 [H] or None."""
-    _need_cuda(qa, positions, seq_of_token, block_table, cache, sink)
+    query in the space of the cache rows; returns sum_j p_j latent_j per head, [T, H*rank].  sink: float32 [H] or None.
+
+    bfloat16 with the transposed latent at hand (vt_cache) and sizes that fit runs the MFMA kernel: for prompts a
+    wave per (token, 16 heads); for a decode step (one token a sequence; max_context bounds the contexts) the keys of
+    every (token, 16 heads) are dealt over several blocks and merged.  Everything else runs the float32 kernel."""
+    _need_cuda(qa, positions, seq_of_token, block_table, cache, sink, vt_cache)
     _rows2d("qa", qa)
     T = qa.shape[0]
     if qa.shape[1] != nheads * (rank + rot):
@@ -762,6 +786,19 @@ def latent_attention(qa: torch.Tensor, positions, seq_of_token, block_table, cac
         raise ValueError(f"the sink is a contiguous float32 [{nheads}] tensor")
     out = torch.empty(T, nheads * rank, dtype=qa.dtype, device=qa.device)
     lib = load()
+    _check_latent_values(vt_cache, cache, rank)
+    if (qa.dtype == torch.bfloat16 and vt_cache is not None and not force_generic and lib.fmsamd_latent_attn_mfma_fits(rank, rot)
+            and qa.stride(0) % 8 == 0):
+        if decode and max_context <= 0:
+            raise ValueError("decode attention needs max_context (an upper bound of every context length)")
+        n_splits = latent_attention_splits(T, nheads, max_context) if decode else 0
+        ws_bytes = lib.fmsamd_latent_attn_workspace(T, nheads, rank, n_splits)
+        ws = torch.empty(max(ws_bytes // 4, 1), dtype=torch.float32, device=qa.device) if ws_bytes else None
+        check(lib.fmsamd_latent_attn_mfma(qa.data_ptr(), qa.stride(0), out.data_ptr(), out.stride(0), _ptr(ws), ws_bytes,
+                                          positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(), block_table.stride(0),
+                                          cache.data_ptr(), vt_cache.data_ptr(), _ptr(sink), T, nheads, rank, rot, float(scale),
+                                          int(window), n_splits, _stream()))
+        return out
     for t0 in range(0, T, 65535):
         n = min(65535, T - t0)
         check(lib.fmsamd_latent_attn_generic(qa[t0:].data_ptr(), qa.stride(0), out[t0:].data_ptr(), out.stride(0), _code(qa.dtype),

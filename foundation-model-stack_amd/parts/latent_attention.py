@@ -67,6 +67,7 @@ class LatentAttention(Mixer):
             self.declare("sink", (nheads,), init="zeros", kind="scale")
         self.o = self.add_child("o", Linear(nheads * vdim, width))
         self._uk_t = self._uv = self._sink = None
+        self._mfma = False  # decided when the model's type is known (finalize)
 
     def fused_parameters(self) -> dict:
         """The fused down-projection as the tensors it is made of, in the order of its rows."""
@@ -75,6 +76,10 @@ class LatentAttention(Mixer):
         return {"down": tuple(pieces)}
 
     def kv_need(self) -> Optional[KVNeed]:
+        """One row [latent | shared key part] per token.  Where the matrix-core kernel runs (bfloat16, sizes that fit
+        it) the latent is kept a second time, transposed, as that kernel's values."""
+        if self._mfma:
+            return KVNeed(1, self.kv_rank + self.rot_dim, self.window, values=True, value_dim=self.kv_rank)
         return KVNeed(1, self.kv_rank + self.rot_dim, self.window, values=False)
 
     @property
@@ -87,6 +92,7 @@ class LatentAttention(Mixer):
 
     def finalize(self, device, dtype) -> None:
         H, D, R, V = self.nheads, self.dim, self.kv_rank, self.vdim
+        self._mfma = dtype == torch.bfloat16 and ops.latent_attention_fits_mfma(R, self.rot_dim) and (H * (R + self.rot_dim)) % 8 == 0
         # Uk_h^T as rows of K = dim contiguous elements: the product that takes a query into the latent space
         self._uk_t = self.w["uk.weight"].view(H, D, R).transpose(1, 2).contiguous()
         self._uv = self.w["uv.weight"].view(H, V, R)
@@ -112,7 +118,7 @@ class LatentAttention(Mixer):
             if not self.owns_kv:
                 raise RuntimeError("this layer has no down-projection for keys and values: it must read another layer's cache")
             ops.latent_kv_write(down, self.kv_col, R, P, self.w["kv_norm.weight"], self.eps, batch.positions, batch.seq_of_token,
-                                table, cos, sin, cache.keys)
+                                table, cos, sin, cache.keys, cache.values)
         cq = ops.rms_norm_cols(down, 0, self.q_rank, self.w["q_norm.weight"], self.eps, x.dtype)
         q = self.uq.forward(cq)
         qa = torch.empty(T, H * (R + P), dtype=x.dtype, device=x.device)
@@ -120,7 +126,8 @@ class LatentAttention(Mixer):
             ops.latent_q_rotate(q, qa, H, D, P, R, batch.positions, cos, sin)
         ops.headwise_linear(q, D + P, self._uk_t, qa, R + P)
         mixed_latent = ops.latent_attention(qa, batch.positions, batch.seq_of_token, table, cache.keys, self._sink, H, R, P,
-                                            self.scale, self.window, decode=batch.is_decode, max_context=batch.context_bound)
+                                            self.scale, self.window, decode=batch.is_decode, max_context=batch.context_bound,
+                                            vt_cache=cache.values)
         mixed = torch.empty(T, H * V, dtype=x.dtype, device=x.device)
         gate = down[:, self.gate_col : self.gate_col + H] if self.has_gate else None
         ops.headwise_linear(mixed_latent, R, self._uv, mixed, V, gate=gate)

@@ -8,9 +8,34 @@ Notation: h is a mixer's or feed-forward's input [T, width]; p_t the position of
 
 from __future__ import annotations
 
+import json
 import math
+import os
 
 import torch
+
+# What a product's or an activation's result is stored as.  Identity for the exact run; a round trip through bfloat16
+# for the run that shows what bfloat16 storage costs (scores, softmax, norms' statistics, the router and the residual
+# sum stay as they are: the design computes them in 32-bit).
+_store = lambda x: x  # noqa: E731
+# When a list: every mixture-of-experts layer appends, per token, by how much the last chosen expert's logit
+# exceeds the best logit not chosen (inf when all experts are chosen).  A small number marks a choice that rounding
+# can turn: such a token's logits are no test of arithmetic.
+router_margins = None
+
+
+def _bf16(x):
+    return x.to(torch.bfloat16).to(x.dtype)
+
+
+def load_model_folder(folder):
+    """(config dictionary, name -> float32 tensor) of a folder with config.json and model.safetensors."""
+    from safetensors.torch import load_file
+
+    with open(os.path.join(folder, "config.json")) as f:
+        config = json.load(f)
+    weights = {k: (v.float() if v.is_floating_point() else v) for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    return config, weights
 
 
 def rms_norm(x, weight, eps):
@@ -39,8 +64,8 @@ def latent_kv(h, w, prefix, m, eps, positions):
     the rotated key part that all heads share [T, rot_dim]."""
     r, rd = m["kv_rank"], m["rot_dim"]
     down = h @ w[prefix + "dkv"].T
-    latent = rms_norm(down[:, :r], w[prefix + "dkv.norm"], eps)
-    shared = rotate_pairs(down[:, r : r + rd], positions, m["rot"]["base"], m["rot"]["dims"])
+    latent = _store(rms_norm(down[:, :r], w[prefix + "dkv.norm"], eps))
+    shared = _store(rotate_pairs(down[:, r : r + rd], positions, m["rot"]["base"], m["rot"]["dims"]))
     return latent, shared
 
 
@@ -49,12 +74,12 @@ def latent_attention(h, w, prefix, m, eps, positions, latent, shared):
     and a gate per head on the output."""
     T = h.shape[0]
     H, d, rd, dv = m["heads"], m["dim"], m["rot_dim"], m["vdim"]
-    cq = rms_norm(h @ w[prefix + "dq"].T, w[prefix + "dq.norm"], eps)
-    q = (cq @ w[prefix + "uq"].T).view(T, H, d + rd)
+    cq = _store(rms_norm(h @ w[prefix + "dq"].T, w[prefix + "dq.norm"], eps))
+    q = _store(cq @ w[prefix + "uq"].T).view(T, H, d + rd)
     q_plain = q[:, :, :d]
-    q_rot = rotate_pairs(q[:, :, d:], positions, m["rot"]["base"], m["rot"]["dims"])
-    k_plain = (latent @ w[prefix + "uk"].T).view(T, H, d)
-    value = (latent @ w[prefix + "uv"].T).view(T, H, dv)
+    q_rot = _store(rotate_pairs(q[:, :, d:], positions, m["rot"]["base"], m["rot"]["dims"]))
+    k_plain = _store(latent @ w[prefix + "uk"].T).view(T, H, d)
+    value = _store(latent @ w[prefix + "uv"].T).view(T, H, dv)
     score = (torch.einsum("thd,shd->hts", q_plain, k_plain) + torch.einsum("thd,sd->hts", q_rot, shared)) * m["scale"]
     visible = positions[None, :] <= positions[:, None]  # [t, s]
     score = score.masked_fill(~visible[None], float("-inf"))
@@ -65,26 +90,29 @@ def latent_attention(h, w, prefix, m, eps, positions, latent, shared):
     prob = e / denom[..., None]
     mixed = torch.einsum("hts,shd->thd", prob, value)
     gate = torch.sigmoid(h @ w[prefix + "g"].T)  # [T, H]
-    mixed = mixed * gate[:, :, None]
-    return mixed.reshape(T, H * dv) @ w[prefix + "o"].T
+    mixed = _store(mixed * gate[:, :, None])
+    return _store(mixed.reshape(T, H * dv) @ w[prefix + "o"].T)
 
 
 def dense_ff(h, w, prefix):
-    z = h @ w[prefix + "up"].T
-    z = 0.5 * z * (1.0 + torch.erf(z / math.sqrt(2.0)))
-    return z @ w[prefix + "down"].T
+    z = _store(h @ w[prefix + "up"].T)
+    z = _store(0.5 * z * (1.0 + torch.erf(z / math.sqrt(2.0))))
+    return _store(z @ w[prefix + "down"].T)
 
 
 def clamped_expert(h, w, prefix, limit):
     g = torch.clamp(h @ w[prefix + "gate"].T, max=limit)
     u = torch.clamp(h @ w[prefix + "up"].T, min=-limit, max=limit)
-    return (g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ w[prefix + "down"].T
+    return _store(g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ w[prefix + "down"].T
 
 
 def moe_ff(h, w, prefix, mlp):
     n, top = mlp["router"]["experts"], mlp["router"]["top"]
     logits = h.float() @ w[prefix + "router"].float().T
     chosen = torch.topk(logits, top, dim=-1)
+    if router_margins is not None:
+        ranked = torch.sort(logits, dim=-1, descending=True).values
+        router_margins.append(ranked[:, top - 1] - ranked[:, top] if top < n else torch.full((h.shape[0],), float("inf")))
     share = torch.softmax(chosen.values, dim=-1).to(h.dtype)
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
@@ -92,13 +120,26 @@ def moe_ff(h, w, prefix, mlp):
             e = int(chosen.indices[t, j])
             out[t] += share[t, j] * clamped_expert(h[t : t + 1], w, f"{prefix}e{e}.", mlp["expert"]["limit"])[0]
     if mlp.get("shared"):
-        s = clamped_expert(h, w, prefix + "shared.", mlp["shared"]["limit"])
+        s = _store(clamped_expert(h, w, prefix + "shared.", mlp["shared"]["limit"]))
         out = out + s * torch.sigmoid(h @ w[prefix + "shared.sg"].T)
-    return out
+    return _store(out)
 
 
-def forward(config, weights, tokens, dtype=torch.float32, return_layers=False):
-    """Logits [T, vocab] of one whole sequence; with return_layers also the stream after every layer."""
+def forward(config, weights, tokens, dtype=torch.float32, return_layers=False, storage=None, margins=None):
+    """Logits [T, vocab] of one whole sequence; with return_layers also the stream after every layer.
+    storage=torch.bfloat16: results of products and activations are rounded to bfloat16 where a bfloat16 model
+    stores them."""
+    global _store, router_margins
+    _store = _bf16 if storage == torch.bfloat16 else (lambda x: x)
+    router_margins = margins  # a list to be filled, or None
+    try:
+        return _forward(config, weights, tokens, dtype, return_layers)
+    finally:
+        _store = lambda x: x  # noqa: E731
+        router_margins = None
+
+
+def _forward(config, weights, tokens, dtype, return_layers):
     w = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in weights.items()}
     eps = config["norm"]["eps"]
     ids = torch.as_tensor(tokens, dtype=torch.long)
@@ -109,7 +150,7 @@ def forward(config, weights, tokens, dtype=torch.float32, return_layers=False):
     for i, layer in enumerate(config["layers"]):
         p = f"l{i}."
         m = layer["mixer"]
-        h = rms_norm(x, w[p + "norm1"], eps)
+        h = _store(rms_norm(x, w[p + "norm1"], eps))
         if layer["type"] != "latent_attention":
             raise ValueError(layer["type"])
         if m.get("kv_from") is None:
@@ -121,9 +162,16 @@ def forward(config, weights, tokens, dtype=torch.float32, return_layers=False):
         x = x + rms_norm(y, w[p + "norm1b"], eps)
         mlp = layer.get("mlp")
         if mlp is not None:
-            h = rms_norm(x, w[p + "norm2"], eps)
+            h = _store(rms_norm(x, w[p + "norm2"], eps))
             y = dense_ff(h, w, p + "mlp.") if mlp["kind"] == "dense" else moe_ff(h, w, p + "mlp.", mlp)
             x = x + rms_norm(y, w[p + "norm2b"], eps)
         after.append(x)
-    logits = rms_norm(x, w["final.norm"], eps) @ w["head"].T
+    logits = _store(rms_norm(x, w["final.norm"], eps)) @ w["head"].T
     return (logits, torch.stack(after)) if return_layers else logits
+
+
+def greedy_generate(config, weights, prompt, n_new):
+    ids = list(prompt)
+    for _ in range(n_new):
+        ids.append(int(forward(config, weights, ids)[-1].argmax()))
+    return ids[len(prompt):]
