@@ -10,6 +10,13 @@ the share of the step's time by kernel class, and further points: decode at batc
 batch 8 with every context near 8000 tokens, the Llama-2-7B shape at batch 8 (256 steps) and the
 Llama-3-70B shape at batch 16 (128 steps).  Decode steps run as generation runs them: the host looks
 at the chosen tokens every `steps_ahead` steps (`--steps-ahead 1`: after every step).
+
+    python bench.py --zodolorn [--layers N]
+
+is another workload (the default one and its record stay as they are): Zodolorn models of a few layer sizes beside
+Llama models of the same width, depth, heads and feed-forward parameters: prefill and decode throughput of both, and
+for every class of kernel its time in one eager prefill and one eager decode step over the time that its bytes and
+flops would take at what this GPU delivers (`x_roofline`: 1 is the roofline).
 """
 
 import argparse
@@ -51,6 +58,8 @@ def main() -> int:
     ap.add_argument("--seq_len", type=int, default=None, help="every prompt of the decode batches has this many tokens")
     ap.add_argument("--batch_size", type=int, default=None, help="the same as --batch")
     ap.add_argument("--max_new_tokens", type=int, default=None, help="the same as --steps: decode steps that are timed")
+    ap.add_argument("--zodolorn", action="store_true",
+                    help="another workload: Zodolorn beside Llama at equal layer sizes, with every kernel class's distance from its roofline")
     args = ap.parse_args()
     if args.seq_len is not None:
         args.prompt_min = args.prompt_max = args.seq_len
@@ -61,6 +70,9 @@ def main() -> int:
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py measures one GPU: this library runs on a single MI355X, --gpus {args.gpus} is not supported")
         return 2
+
+    if args.zodolorn:
+        return zodolorn_comparison(args)
 
     import torch
 
@@ -282,6 +294,180 @@ def main() -> int:
         "shares": shares,
         "points": points,
     }
+    print(json.dumps(record))
+    return 0
+
+
+# ---- Zodolorn beside Llama ------------------------------------------------------------------------------------------
+# (name, width, heads, [dim, rot, vdim, q_rank, kv_rank], dense ff, experts, top, expert ff, shared ff, vocabulary)
+ZODOLORN_SIZES = [
+    ("w2048", 2048, 16, (128, 64, 128, 768, 512), 8192, 32, 4, 1024, 2048, 32768),
+    ("w4096", 4096, 32, (128, 64, 128, 1536, 512), 12288, 64, 6, 1536, 3072, 32768),
+]
+
+
+def zodolorn_comparison(args) -> int:
+    import torch
+
+    import fms_amd
+    from fms_amd.architectures.zodolorn import make_config
+    from fms_amd.engine import Engine
+    from fms_amd.kernels import ops
+    from fms_amd.sampling import SamplingParams, choose
+
+    read_bps, mfma_flops = ops.measured_peaks()
+    greedy = SamplingParams(do_sample=False)
+    rng = random.Random(args.seed)
+    layers = args.layers or 4
+    context = 8192
+
+    # bytes and flops of one call of an op, from its arguments (weights and caches are read once, activations once)
+    # keys_read: the sum over the step's tokens of the keys each of them sees (flops); keys_loaded: the keys that have to
+    # come from memory at least once (a prompt's keys serve all its queries; a decode step reads every context once)
+    state = {"keys_read": 0, "keys_loaded": 0}
+
+    def nbytes(*tensors):
+        return sum(t.numel() * t.element_size() for t in tensors if t is not None)
+
+    def cost(name, a, kw, out):
+        if name in ("linear", "gated_linear", "linear_into_stream"):
+            x, w = a[0], a[1]
+            return nbytes(x, w) + (nbytes(out) if torch.is_tensor(out) else 0), 2.0 * x.shape[0] * w.shape[0] * w.shape[1]
+        if name == "headwise_linear":
+            x, w, y = a[0], a[2], a[3]
+            return nbytes(w) + 2 * x.shape[0] * w.shape[0] * (w.shape[1] + w.shape[2]), 2.0 * x.shape[0] * w.numel()
+        if name == "attention":  # grouped-query attention over keys and values of kvheads x head_dim
+            H, K, D = a[6], a[7], a[8]
+            return 2 * state["keys_loaded"] * 2 * K * D + 2 * nbytes(a[0][:, : H * D]), 4.0 * state["keys_read"] * H * D
+        if name == "latent_attention":  # one row of rank + rot a key, and the latent once more as values
+            H, R, P = a[6], a[7], a[8]
+            return 2 * state["keys_loaded"] * (2 * R + P) + nbytes(a[0]) + 2 * a[0].shape[0] * H * R, 2.0 * state["keys_read"] * H * (2 * R + P)
+        if name == "moe_experts":
+            x, ids, g, u, d = a[:5]
+            used = min(g.shape[0], ids.numel())  # experts whose weights are read at least once
+            return used * (nbytes(g, u, d) // g.shape[0]) + ids.numel() * (2 * x.shape[1] * x.element_size() + 4 * x.shape[1]), 6.0 * ids.numel() * g.shape[1] * g.shape[2]
+        tensors = [t for t in a if torch.is_tensor(t)] + ([out] if torch.is_tensor(out) else [])
+        return nbytes(*[t for t in tensors if t.dim() == 2 and t.shape[0] == tensors[0].shape[0]]), 0.0
+
+    watched = ["linear", "gated_linear", "linear_into_stream", "headwise_linear", "attention", "latent_attention", "moe_experts",
+               "moe_route", "moe_combine", "add_norm", "norm_add_norm", "rms_norm_cols", "rope_kv_write", "qkv_rope_write",
+               "latent_kv_write", "latent_q_rotate", "activation", "clamped_gated_act", "gated_act", "embed"]
+    small = {"moe_route", "moe_combine", "add_norm", "norm_add_norm", "rms_norm_cols", "rope_kv_write", "latent_kv_write",
+             "latent_q_rotate", "activation", "clamped_gated_act", "gated_act", "embed"}
+
+    def classes_of_a_step(run):
+        """{class: (ms, ms at the roofline)} of the kernels of `run()`, by events around every call into the library."""
+        spans, originals = [], {}
+
+        def timed(name, fn):
+            def call(*a, **kw):
+                first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                first.record()
+                out = fn(*a, **kw)
+                last.record()
+                b, f = cost(name, a, kw, out)
+                spans.append(("elementwise" if name in small else name, first, last, b, f))
+                return out
+            return call
+
+        for name in watched:
+            originals[name] = getattr(ops, name)
+            setattr(ops, name, timed(name, originals[name]))
+        try:
+            run()
+            torch.cuda.synchronize()
+        finally:
+            for name, fn in originals.items():
+                setattr(ops, name, fn)
+        out = {}
+        for kind, first, last, b, f in spans:
+            ms, ideal = out.get(kind, (0.0, 0.0))
+            out[kind] = (ms + first.elapsed_time(last), ideal + 1000 * max(b / read_bps, f / mfma_flops))
+        return {k: {"ms": round(ms, 4), "x_roofline": round(ms / ideal, 2) if ideal else None} for k, (ms, ideal) in sorted(out.items())}
+
+    def measure(model, vocab):
+        out = {}
+        for n in (512, 2048):
+            engine = Engine(model, max_tokens=n + 64, max_slots=1, use_graphs=False)
+            times = []
+            for i in range(4):
+                slot = engine.new_sequence()
+                ids = [rng.randrange(vocab) for _ in range(n)]
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                engine.step([slot], [ids], "last")
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t0)
+                engine.end_sequence(slot)
+            t = sorted(times[1:])[1]
+            out[f"prefill_{n}_tok_s"] = round(n / t, 1)
+            out[f"prefill_{n}_ms"] = round(1000 * t, 3)
+            if n == 2048:
+                slot = engine.new_sequence()
+                state.update(keys_read=n * (n + 1) // 2, keys_loaded=n)
+                out["prefill_2048_kernels"] = classes_of_a_step(lambda: engine.step([slot], [ids], "last"))
+                engine.end_sequence(slot)
+            del engine
+        for batch, prompt in ((1, 1024), (8, 1024), (64, 1024), (8, 7000)):
+            steps, warmup = 32, 4
+            lens = [rng.randint(prompt // 2, prompt) for _ in range(batch)]
+            room = sum(-(-(n + steps + warmup + 16) // 64) * 64 for n in lens)
+            engine = Engine(model, max_tokens=room, max_slots=batch)
+            slots = [engine.new_sequence() for _ in range(batch)]
+            tokens = []
+            for b in range(batch):
+                logits = engine.step([slots[b]], [[rng.randrange(vocab) for _ in range(lens[b])]], "last")
+                tokens += choose(logits, greedy).tolist()
+
+            def run(n):
+                nonlocal tokens
+                done = 0
+                while done < n:
+                    ahead = min(4, n - done)
+                    tokens = engine.decode_and_choose_many(slots, tokens, greedy, steps=ahead)[-1]
+                    done += ahead
+
+            run(warmup)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            run(steps)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            name = f"decode_b{batch}_ctx{prompt}"
+            out[f"{name}_tok_s"] = round(batch * steps / dt, 1)
+            out[f"{name}_ms"] = round(1000 * dt / steps, 3)
+            if (batch, prompt) in ((8, 1024), (8, 7000)):
+                state.update(keys_read=sum(lens) + batch * (warmup + steps + 1), keys_loaded=sum(lens) + batch * (warmup + steps + 1))
+                out[f"{name}_kernels"] = classes_of_a_step(lambda: engine.step(slots, [[t] for t in tokens], "last"))
+            for s in slots:
+                engine.end_sequence(s)
+            del engine
+            torch.cuda.empty_cache()
+        return out
+
+    record = {"workload": "zodolorn beside llama at equal layer sizes", "layers": layers, "dtype": "bf16",
+              "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
+              "peak_measured": {"read_gbs": round(read_bps / 1e9, 1), "mfma_tflops": round(mfma_flops / 1e12, 1)}, "sizes": {}}
+    for name, width, heads, (dim, rot, vdim, q_rank, kv_rank), dense_ff, experts, top, expert_ff, shared_ff, vocab in ZODOLORN_SIZES:
+        config = make_config(width=width, vocab=vocab, nlayers=layers, heads=heads, dim=dim, rot_dim=rot, vdim=vdim, q_rank=q_rank,
+                             kv_rank=kv_rank, dense_ff=dense_ff, experts=experts, top=top, expert_ff=expert_ff, shared_ff=shared_ff,
+                             max_positions=context)
+        model = fms_amd.from_config(config, "zodolorn", data_type="bf16", random_seed=args.seed)
+        mine = measure(model, vocab)
+        del model
+        torch.cuda.empty_cache()
+        # Llama of the same width, depth and heads; its gated feed-forward has the parameters of the plain one (2/3 of its width)
+        hidden = -(-dense_ff * 2 // 3 // 256) * 256
+        llama = fms_amd.get_model("llama", "micro", data_type="bf16", random_seed=args.seed, emb_dim=width, nheads=heads, kvheads=8,
+                                  nlayers=layers, hidden_dim=hidden, src_vocab_size=vocab, max_expected_seq_len=context)
+        theirs = measure(llama, vocab)
+        del llama
+        torch.cuda.empty_cache()
+        record["sizes"][name] = {"zodolorn": dict(config=dict(width=width, heads=heads, dim=dim, rot_dim=rot, vdim=vdim, q_rank=q_rank,
+                                                                kv_rank=kv_rank, dense_ff=dense_ff, experts=experts, top=top,
+                                                                expert_ff=expert_ff, shared_ff=shared_ff, vocab=vocab), **mine),
+                                 "llama": dict(config=dict(width=width, heads=heads, kvheads=8, head_dim=width // heads, hidden=hidden,
+                                                           vocab=vocab), **theirs)}
     print(json.dumps(record))
     return 0
 

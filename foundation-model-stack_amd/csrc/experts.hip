@@ -193,7 +193,7 @@ __global__ void __launch_bounds__(TILE_THREADS) expert_gate_up_mfma_kernel(Exper
   const bf16* wg = (const bf16*)a.w1 + (size_t)e * a.N * a.K;
   const bf16* wu = (const bf16*)a.w2 + (size_t)e * a.N * a.K;
   auto a_row = [&](int m) { return m < rows ? x + (size_t)(a.order[start + m] / a.top) * a.ldx : (const bf16*)nullptr; };
-  f32x4 g[4], u[4];
+  f32x4 g[TILE_MFMA_WAVE_TILES], u[TILE_MFMA_WAVE_TILES];
   tile_product_mfma(a_row, [&](int n) { return n0 + n < a.N ? wg + (size_t)(n0 + n) * a.K : (const bf16*)nullptr; }, a.K, g);
   tile_product_mfma(a_row, [&](int n) { return n0 + n < a.N ? wu + (size_t)(n0 + n) * a.K : (const bf16*)nullptr; }, a.K, u);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -202,8 +202,8 @@ __global__ void __launch_bounds__(TILE_THREADS) expert_gate_up_mfma_kernel(Exper
     const int m = (lane >> 4) * 4 + i;
     if (m >= rows) continue;
 #pragma unroll
-    for (int tl = 0; tl < 4; ++tl) {
-      const int n = n0 + wave * 64 + tl * 16 + (lane & 15);
+    for (int tl = 0; tl < TILE_MFMA_WAVE_TILES; ++tl) {
+      const int n = n0 + wave * (16 * TILE_MFMA_WAVE_TILES) + tl * 16 + (lane & 15);
       if (n < a.N) ((bf16*)a.y)[(size_t)(start + m) * a.N + n] = (bf16)clamp_gated(g[tl][i], u[tl][i], a.limit, a.alpha, a.shift);
     }
   }
@@ -215,7 +215,7 @@ __global__ void __launch_bounds__(TILE_THREADS) expert_down_mfma_kernel(ExpertAr
   const int n0 = blockIdx.y * TILE_MFMA_COLS;
   const bf16* x = (const bf16*)a.x;
   const bf16* w = (const bf16*)a.w1 + (size_t)e * a.N * a.K;
-  f32x4 acc[4];
+  f32x4 acc[TILE_MFMA_WAVE_TILES];
   tile_product_mfma([&](int m) { return m < rows ? x + (size_t)(start + m) * a.ldx : (const bf16*)nullptr; },
                     [&](int n) { return n0 + n < a.N ? w + (size_t)(n0 + n) * a.K : (const bf16*)nullptr; }, a.K, acc);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -225,8 +225,8 @@ __global__ void __launch_bounds__(TILE_THREADS) expert_down_mfma_kernel(ExpertAr
     if (m >= rows) continue;
     float* yrow = (float*)a.y + (size_t)a.order[start + m] * a.N;
 #pragma unroll
-    for (int tl = 0; tl < 4; ++tl) {
-      const int n = n0 + wave * 64 + tl * 16 + (lane & 15);
+    for (int tl = 0; tl < TILE_MFMA_WAVE_TILES; ++tl) {
+      const int n = n0 + wave * (16 * TILE_MFMA_WAVE_TILES) + tl * 16 + (lane & 15);
       if (n < a.N) yrow[n] = acc[tl][i];
     }
   }

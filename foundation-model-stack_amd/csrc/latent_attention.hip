@@ -162,7 +162,7 @@ __global__ void __launch_bounds__(TILE_THREADS) headwise_mfma_kernel(HeadwiseArg
   const int t0 = blockIdx.x * TILE_ROWS, h = blockIdx.y, n0 = blockIdx.z * TILE_MFMA_COLS;
   const bf16* x = (const bf16*)a.x + (size_t)h * a.xs;
   const bf16* w = (const bf16*)a.w + (size_t)h * a.N * a.K;
-  f32x4 acc[4];
+  f32x4 acc[TILE_MFMA_WAVE_TILES];
   tile_product_mfma([&](int m) { return t0 + m < a.T ? x + (size_t)(t0 + m) * a.ldx : (const bf16*)nullptr; },
                     [&](int n) { return n0 + n < a.N ? w + (size_t)(n0 + n) * a.K : (const bf16*)nullptr; }, a.K, acc);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -172,8 +172,8 @@ __global__ void __launch_bounds__(TILE_THREADS) headwise_mfma_kernel(HeadwiseArg
     if (t >= a.T) continue;
     const float g = a.gate ? 1.f / (1.f + expf(-a.gate[(size_t)t * a.ldg + h])) : 1.f;
 #pragma unroll
-    for (int tl = 0; tl < 4; ++tl) {
-      const int n = n0 + wave * 64 + tl * 16 + (lane & 15);
+    for (int tl = 0; tl < TILE_MFMA_WAVE_TILES; ++tl) {
+      const int n = n0 + wave * (16 * TILE_MFMA_WAVE_TILES) + tl * 16 + (lane & 15);
       if (n < a.N) ((bf16*)a.y)[(size_t)t * a.ldy + (size_t)h * a.ys + n] = (bf16)(acc[tl][i] * g);
     }
   }
@@ -323,15 +323,124 @@ extern "C" int fmsamd_latent_attn_generic(const void* qa, long ldq, void* out, l
 // --------------------------------------------------------------------------
 #define LAT_EMPTY -1e30f
 
+// The state of a wave's 16 columns, and one tile of 32 keys worked into it.  load_k(which, c) gives this lane's eight
+// elements c * 32 + grp * 8 .. of its row of score tile a (which 0) or b (1); load_v(dt) its eight keys grp * 8 .. of
+// latent element dt * 16 + col.  Loads are asked for in groups (KG steps of K, VG tiles of the latent) before the
+// first of a group is multiplied: with the accumulators of a large latent a wave has a SIMD to itself, and the loads
+// it keeps in flight are all that hides the memory's latency.
 template <int RT, int WC>
+struct LatentState {
+  f32x4 acc[RT];
+  float m, l;
+};
+
+template <int RT, int WC, typename LoadQ, typename LoadK, typename LoadV>
+__device__ __forceinline__ void latent_tile(LatentState<RT, WC>& st, LoadQ load_q, LoadK load_k, LoadV load_v, int base,
+                                            int lo, int pos, int rank, int width, float scale, int grp) {
+  constexpr int KG = WC <= 10 ? WC : 6;
+  constexpr int VG = RT <= 16 ? RT : 8;
+  f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int c0 = 0; c0 < WC; c0 += KG) {
+    bf16x8 ka[KG], kb[KG];
+#pragma unroll
+    for (int c = 0; c < KG; ++c) {
+      if (c0 + c < WC && (c0 + c) * 32 < width) ka[c] = load_k(0, c0 + c), kb[c] = load_k(1, c0 + c);
+    }
+#pragma unroll
+    for (int c = 0; c < KG; ++c) {
+      if (c0 + c < WC && (c0 + c) * 32 < width) {
+        const bf16x8 q = load_q(c0 + c);
+        sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[c], q, sa, 0, 0, 0);
+        sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb[c], q, sb, 0, 0, 0);
+      }
+    }
+  }
+  // this lane's scores: keys base + 8 grp + i (sa) and base + 8 grp + 4 + i (sb) of its column
+  float s[8];
+  float top = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int ja = base + 8 * grp + i, jb = ja + 4;
+    s[i] = (ja >= lo && ja <= pos) ? sa[i] * scale : -INFINITY;
+    s[4 + i] = (jb >= lo && jb <= pos) ? sb[i] * scale : -INFINITY;
+    top = fmaxf(top, fmaxf(s[i], s[4 + i]));
+  }
+  top = fmaxf(top, __shfl_xor(top, 16, WAVE));
+  top = fmaxf(top, __shfl_xor(top, 32, WAVE));
+  const float m_new = fmaxf(st.m, top);
+  const float alpha = __expf(st.m - m_new);
+  float psum = 0.f;
+  bf16x8 pmat;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float p = __expf(s[i] - m_new);  // exp(-inf) = 0 for the keys that are not seen
+    psum += p;
+    pmat[i] = (bf16)p;
+  }
+  st.l = st.l * alpha + psum;
+  st.m = m_new;
+#pragma unroll
+  for (int d0 = 0; d0 < RT; d0 += VG) {
+    bf16x8 v[VG];
+#pragma unroll
+    for (int dt = 0; dt < VG; ++dt) {
+      if (d0 + dt < RT && (d0 + dt) * 16 < rank) v[dt] = load_v(d0 + dt);
+    }
+#pragma unroll
+    for (int dt = 0; dt < VG; ++dt) {
+      if (d0 + dt < RT && (d0 + dt) * 16 < rank) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) st.acc[d0 + dt][i] *= alpha;
+        st.acc[d0 + dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v[dt], pmat, st.acc[d0 + dt], 0, 0, 0);
+      }
+    }
+  }
+}
+
+// What a wave leaves: the normalised result (one part) or its part's maximum, sum and unnormalised result.
+template <int RT, int WC>
+__device__ __forceinline__ void latent_finish(LatentState<RT, WC>& st, bf16* __restrict__ out, long ldo, float* __restrict__ ws, int t,
+                                              int head, int nheads, int rank, int n_parts, int part, int grp) {
+  st.l += __shfl_xor(st.l, 16, WAVE);
+  st.l += __shfl_xor(st.l, 32, WAVE);
+  if (head >= nheads) return;
+  // acc[dt][i] is element d = dt * 16 + grp * 4 + i of this lane's column
+  if (n_parts == 1) {
+    const float inv = st.l > 0.f ? 1.f / st.l : 0.f;
+    bf16* o = out + (size_t)t * ldo + (size_t)head * rank;
+#pragma unroll
+    for (int dt = 0; dt < RT; ++dt) {
+      if (dt * 16 < rank) {
+        bf16x4 r = {(bf16)(st.acc[dt][0] * inv), (bf16)(st.acc[dt][1] * inv), (bf16)(st.acc[dt][2] * inv), (bf16)(st.acc[dt][3] * inv)};
+        *reinterpret_cast<bf16x4*>(o + dt * 16 + grp * 4) = r;
+      }
+    }
+  } else {
+    float* w = ws + (((size_t)t * nheads + head) * n_parts + part) * (rank + 4);
+    if (grp == 0) w[0] = st.m, w[1] = st.l;
+#pragma unroll
+    for (int dt = 0; dt < RT; ++dt) {
+      if (dt * 16 < rank) *reinterpret_cast<f32x4*>(w + 4 + dt * 16 + grp * 4) = st.acc[dt];
+    }
+  }
+}
+
+// LDS: the four waves of a block (four consecutive tiles of one sequence: neighbouring tokens, or the head groups of
+// one token) share every tile of keys through LDS, so a tile comes from the caches once a block instead of once a
+// wave; a block whose tiles lie in different sequences, and every block of a decode step, loads straight from
+// global memory.
+template <int RT, int WC, bool LDS>
 __global__ void __launch_bounds__(256)
     latent_attn_mfma_kernel(const bf16* __restrict__ qa, long ldq, bf16* __restrict__ out, long ldo, float* __restrict__ ws,
                             const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                             const int* __restrict__ block_table, int table_stride, const bf16* __restrict__ cache,
                             const bf16* __restrict__ vt_cache, const float* __restrict__ sink, int n_tokens, int nheads,
                             int rank, int width, float scale, int window, int tiles_per_token, int n_parts) {
+  extern __shared__ __attribute__((aligned(16))) bf16 lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, grp = lane >> 4;
+  const int n_tiles = n_tokens * tiles_per_token;
   int tile, part;
   if (n_parts == 1) {
     tile = blockIdx.x * 4 + wave;
@@ -340,118 +449,140 @@ __global__ void __launch_bounds__(256)
     tile = blockIdx.x;
     part = blockIdx.y * 4 + wave;
   }
-  if (tile >= n_tokens * tiles_per_token) return;
-  const int t = tile / tiles_per_token;
-  const int head = (tile % tiles_per_token) * 16 + col;
-  const bool valid = head < nheads;
-  const int seq = uniform_load(seq_of_token + t);
-  if (seq < 0) {
-    if (n_parts == 1 && valid) {
-      for (int d = grp; d < rank; d += 4) out[(size_t)t * ldo + (size_t)head * rank + d] = (bf16)0.f;
-    }
-    return;
+  // do the block's four tiles share their keys?  (every wave works that out for itself, and all agree)
+  bool together = false;
+  int seq = -1, pos = -1, t = 0;
+  if (tile < n_tiles) {
+    t = tile / tiles_per_token;
+    seq = uniform_load(seq_of_token + t);
+    pos = seq >= 0 ? uniform_load(positions + t) : -1;
   }
-  const int pos = uniform_load(positions + t);
+  int first_pos = 0x7fffffff, last_pos = -1;
+  if (LDS) {
+    together = true;
+    int common = -2;
+    for (int w = 0; w < 4; ++w) {
+      const int tl = blockIdx.x * 4 + w;
+      if (tl >= n_tiles) continue;
+      const int tt = tl / tiles_per_token;
+      const int sq = uniform_load(seq_of_token + tt);
+      if (sq < 0) continue;
+      if (common == -2) common = sq;
+      together = together && sq == common;
+      const int p = uniform_load(positions + tt);
+      first_pos = p < first_pos ? p : first_pos;
+      last_pos = p > last_pos ? p : last_pos;
+    }
+    together = together && common >= 0;
+  }
+  const int head = (tile % tiles_per_token) * 16 + col;
+  const bool valid = tile < n_tiles && seq >= 0 && head < nheads;
+  if (!(LDS && together)) {
+    if (tile >= n_tiles) return;
+    if (seq < 0) {
+      if (n_parts == 1 && head < nheads) {
+        for (int d = grp; d < rank; d += 4) out[(size_t)t * ldo + (size_t)head * rank + d] = (bf16)0.f;
+      }
+      return;
+    }
+  }
   const int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
-  const int* bt = block_table + (size_t)seq * table_stride;
 
+  // The wave's queries wait in LDS, each lane's eight elements of every step of K in a slot of its own (written and
+  // read by the same lane: no barrier): in registers they would crowd out the loads that have to be in flight.
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-  bf16x8 qreg[WC];
+  bf16* q_lds = lds + ((size_t)wave * WC * 64 + lane) * 8;
   {
     const bf16* qrow = qa + (size_t)t * ldq + (size_t)(valid ? head : 0) * width;
 #pragma unroll
     for (int c = 0; c < WC; ++c) {
       const int k = c * 32 + grp * 8;
-      qreg[c] = (valid && k < width) ? *reinterpret_cast<const bf16x8*>(qrow + k) : zero8;
+      *reinterpret_cast<bf16x8*>(q_lds + c * 64 * 8) = (valid && k < width) ? *reinterpret_cast<const bf16x8*>(qrow + k) : zero8;
     }
   }
-  f32x4 acc[RT];
+  auto load_q = [&](int c) { return *reinterpret_cast<const bf16x8*>(q_lds + c * 64 * 8); };
+  LatentState<RT, WC> st;
 #pragma unroll
-  for (int dt = 0; dt < RT; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m_run = (sink && valid) ? sink[head] : LAT_EMPTY;
-  float l_run = (sink && valid && part == 0 && grp == 0) ? 1.f : 0.f;
-
+  for (int dt = 0; dt < RT; ++dt) st.acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  st.m = (sink && valid) ? sink[head] : LAT_EMPTY;
+  st.l = (sink && valid && part == 0 && grp == 0) ? 1.f : 0.f;
   const int key_a = 8 * (col >> 2) + (col & 3);  // the key of this lane's row in score tile a; tile b: + 4
-  for (int kt = lo / 32 + part; kt * 32 <= pos; kt += n_parts) {
-    const int base = kt * 32;
-    const size_t page = readable_page(uniform_load(bt + base / PAGE_TOKENS));
-    const int in_page = base % PAGE_TOKENS;
-    const bf16* ka = cache + (page * PAGE_TOKENS + in_page + key_a) * width + grp * 8;
-    const bf16* kb = ka + 4 * (size_t)width;
-    f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int c = 0; c < WC; ++c) {
-      if (c * 32 < width) {
-        const bool in = c * 32 + grp * 8 < width;
-        const bf16x8 a = in ? *reinterpret_cast<const bf16x8*>(ka + c * 32) : zero8;
-        const bf16x8 b = in ? *reinterpret_cast<const bf16x8*>(kb + c * 32) : zero8;
-        sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qreg[c], sa, 0, 0, 0);
-        sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b, qreg[c], sb, 0, 0, 0);
+
+  if (LDS && together) {
+    // all four waves walk the keys that any of them sees; a wave's own mask hides what it must not see
+    const int ks = width + 8, vs = 32 + 8;  // row strides in LDS (elements): 16 bytes of padding against bank conflicts
+    bf16* k_lds = lds + 4 * WC * 64 * 8;  // behind the four waves' queries
+    bf16* v_lds = k_lds + 32 * ks;
+    const int first_lo = window > 0 ? (first_pos - window + 1 > 0 ? first_pos - window + 1 : 0) : 0;
+    const int common_seq = uniform_load(seq_of_token + (blockIdx.x * 4 < n_tiles ? (blockIdx.x * 4) / tiles_per_token : 0));
+    int any_seq = common_seq;
+    if (any_seq < 0) any_seq = seq;  // the block's first tile may be a padding row
+    for (int w = 0; w < 4 && any_seq < 0; ++w) {
+      const int tl = blockIdx.x * 4 + w;
+      if (tl < n_tiles) any_seq = uniform_load(seq_of_token + tl / tiles_per_token);
+    }
+    const int* bt = block_table + (size_t)any_seq * table_stride;
+    const int chunks_k = width / 8;  // 16-byte pieces in a key row
+    for (int base = (first_lo / 32) * 32; base <= last_pos; base += 32) {
+      const size_t page = readable_page(uniform_load(bt + base / PAGE_TOKENS));
+      const int in_page = base % PAGE_TOKENS;
+      __syncthreads();  // the tile before this one has been read by every wave
+      for (int i = threadIdx.x; i < 32 * chunks_k; i += 256) {
+        const int r = i / chunks_k, ch = i % chunks_k;
+        *reinterpret_cast<bf16x8*>(k_lds + r * ks + ch * 8) =
+            *reinterpret_cast<const bf16x8*>(cache + (page * PAGE_TOKENS + in_page + r) * width + ch * 8);
+      }
+      for (int i = threadIdx.x; i < rank * 4; i += 256) {
+        const int d = i >> 2, ch = i & 3;
+        *reinterpret_cast<bf16x8*>(v_lds + d * vs + ch * 8) =
+            *reinterpret_cast<const bf16x8*>(vt_cache + (page * rank + d) * PAGE_TOKENS + in_page + ch * 8);
+      }
+      __syncthreads();
+      // (a condition that all lanes of the wave share: matrix instructions take their operands from every lane)
+      if (tile < n_tiles && seq >= 0 && base <= pos) {
+        latent_tile<RT, WC>(
+            st, load_q,
+            [&](int which, int c) {
+              return c * 32 + grp * 8 < width ? *reinterpret_cast<const bf16x8*>(k_lds + (key_a + 4 * which) * ks + c * 32 + grp * 8) : zero8;
+            },
+            [&](int dt) { return *reinterpret_cast<const bf16x8*>(v_lds + (dt * 16 + col) * vs + grp * 8); }, base, lo, pos, rank, width,
+            scale, grp);
       }
     }
-    // this lane's scores: keys base + 8 grp + i (sa) and base + 8 grp + 4 + i (sb) of column `col`
-    float s[8];
-    float top = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int ja = base + 8 * grp + i, jb = ja + 4;
-      s[i] = (ja >= lo && ja <= pos) ? sa[i] * scale : -INFINITY;
-      s[4 + i] = (jb >= lo && jb <= pos) ? sb[i] * scale : -INFINITY;
-      top = fmaxf(top, fmaxf(s[i], s[4 + i]));
-    }
-    top = fmaxf(top, __shfl_xor(top, 16, WAVE));
-    top = fmaxf(top, __shfl_xor(top, 32, WAVE));
-    const float m_new = fmaxf(m_run, top);
-    const float alpha = __expf(m_run - m_new);
-    float psum = 0.f;
-    bf16x8 pmat;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const float p = __expf(s[i] - m_new);  // exp(-inf) = 0 for the keys that are not seen
-      psum += p;
-      pmat[i] = (bf16)p;
-    }
-    l_run = l_run * alpha + psum;
-    m_run = m_new;
-    const bf16* vt = vt_cache + (page * rank + col) * PAGE_TOKENS + in_page + grp * 8;
-#pragma unroll
-    for (int dt = 0; dt < RT; ++dt) {
-      if (dt * 16 < rank) {
-        const bf16x8 v = *reinterpret_cast<const bf16x8*>(vt + (size_t)dt * 16 * PAGE_TOKENS);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc[dt][i] *= alpha;
-        acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pmat, acc[dt], 0, 0, 0);
+    if (tile >= n_tiles) return;
+    if (seq < 0) {
+      if (head < nheads) {
+        for (int d = grp; d < rank; d += 4) out[(size_t)t * ldo + (size_t)head * rank + d] = (bf16)0.f;
       }
-    }
-  }
-  l_run += __shfl_xor(l_run, 16, WAVE);
-  l_run += __shfl_xor(l_run, 32, WAVE);
-  if (!valid) return;
-  // acc[dt][i] is element d = dt * 16 + grp * 4 + i of column `col`
-  if (n_parts == 1) {
-    const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
-    bf16* o = out + (size_t)t * ldo + (size_t)head * rank;
-#pragma unroll
-    for (int dt = 0; dt < RT; ++dt) {
-      if (dt * 16 < rank) {
-        bf16x4 r = {(bf16)(acc[dt][0] * inv), (bf16)(acc[dt][1] * inv), (bf16)(acc[dt][2] * inv), (bf16)(acc[dt][3] * inv)};
-        *reinterpret_cast<bf16x4*>(o + dt * 16 + grp * 4) = r;
-      }
+      return;
     }
   } else {
-    float* w = ws + (((size_t)t * nheads + head) * n_parts + part) * (rank + 4);
-    if (grp == 0) w[0] = m_run, w[1] = l_run;
-#pragma unroll
-    for (int dt = 0; dt < RT; ++dt) {
-      if (dt * 16 < rank) *reinterpret_cast<f32x4*>(w + 4 + dt * 16 + grp * 4) = acc[dt];
+    const int* bt = block_table + (size_t)seq * table_stride;
+    for (int kt = lo / 32 + part; kt * 32 <= pos; kt += n_parts) {
+      const int base = kt * 32;
+      const size_t page = readable_page(uniform_load(bt + base / PAGE_TOKENS));
+      const int in_page = base % PAGE_TOKENS;
+      const bf16* ka = cache + (page * PAGE_TOKENS + in_page + key_a) * width + grp * 8;
+      const bf16* vt = vt_cache + (page * rank + col) * PAGE_TOKENS + in_page + grp * 8;
+      latent_tile<RT, WC>(
+          st, load_q,
+          [&](int which, int c) {
+            return c * 32 + grp * 8 < width ? *reinterpret_cast<const bf16x8*>(ka + which * 4 * (size_t)width + c * 32) : zero8;
+          },
+          [&](int dt) { return *reinterpret_cast<const bf16x8*>(vt + (size_t)dt * 16 * PAGE_TOKENS); }, base, lo, pos, rank, width, scale,
+          grp);
     }
   }
+  latent_finish<RT, WC>(st, out, ldo, ws, t, head, nheads, rank, n_parts, part, grp);
 }
 
-// out[t, h, :] = sum_i acc_i exp(m_i - M) / sum_i l_i exp(m_i - M) over the parts i
+// out[t, h, :] = sum_i acc_i exp(m_i - M) / sum_i l_i exp(m_i - M) over the parts i.  The parts' maxima and sums are
+// loaded side by side (a thread a part) and their weights left in LDS: no chain of dependent loads.
+#define LAT_MAX_PARTS 256
 __global__ void __launch_bounds__(64)
     latent_attn_merge_kernel(const float* __restrict__ ws, bf16* __restrict__ out, long ldo, const int* __restrict__ seq_of_token,
                              int nheads, int rank, int n_parts) {
+  __shared__ float weight[LAT_MAX_PARTS];
   const int h = blockIdx.x, t = blockIdx.y;
   bf16* o = out + (size_t)t * ldo + (size_t)h * rank;
   if (seq_of_token[t] < 0) {
@@ -460,13 +591,21 @@ __global__ void __launch_bounds__(64)
   }
   const float* w = ws + ((size_t)t * nheads + h) * n_parts * (rank + 4);
   float top = LAT_EMPTY;
-  for (int i = 0; i < n_parts; ++i) top = fmaxf(top, w[(size_t)i * (rank + 4)]);
+  for (int i = threadIdx.x; i < n_parts; i += WAVE) top = fmaxf(top, w[(size_t)i * (rank + 4)]);
+  top = wave_max(top);
   float total = 0.f;
-  for (int i = 0; i < n_parts; ++i) total += w[(size_t)i * (rank + 4) + 1] * __expf(w[(size_t)i * (rank + 4)] - top);
+  for (int i = threadIdx.x; i < n_parts; i += WAVE) {
+    const float e = __expf(w[(size_t)i * (rank + 4)] - top);
+    weight[i] = e;
+    total += w[(size_t)i * (rank + 4) + 1] * e;
+  }
+  total = wave_sum(total);
+  __syncthreads();
   const float inv = total > 0.f ? 1.f / total : 0.f;
   for (int d = threadIdx.x; d < rank; d += blockDim.x) {
     float v = 0.f;
-    for (int i = 0; i < n_parts; ++i) v = fmaf(w[(size_t)i * (rank + 4) + 4 + d], __expf(w[(size_t)i * (rank + 4)] - top), v);
+#pragma unroll 8
+    for (int i = 0; i < n_parts; ++i) v = fmaf(w[(size_t)i * (rank + 4) + 4 + d], weight[i], v);
     o[d] = (bf16)(v * inv);
   }
 }
@@ -494,7 +633,7 @@ extern "C" int fmsamd_latent_attn_mfma(const void* qa, long ldq, void* out, long
               n_tokens, nheads, rank, rot);
   FMS_REQUIRE(ldq >= (long)nheads * width && ldq % 8 == 0 && ldo >= (long)nheads * rank && ldo % 4 == 0 && ((uintptr_t)qa % 16) == 0,
               "latent_attn_mfma: rows too short or not aligned");
-  FMS_REQUIRE(cache != nullptr && vt_cache != nullptr && window >= 0 && n_splits >= 0 && n_splits <= 16384, "latent_attn_mfma: bad arguments");
+  FMS_REQUIRE(cache != nullptr && vt_cache != nullptr && window >= 0 && n_splits >= 0 && n_splits * 4 <= LAT_MAX_PARTS, "latent_attn_mfma: bad arguments (at most 64 splits)");
   const int tiles_per_token = ceil_div(nheads, 16);
   const long tiles = (long)n_tokens * tiles_per_token;
   const int n_parts = n_splits == 0 ? 1 : n_splits * 4;
@@ -502,14 +641,39 @@ extern "C" int fmsamd_latent_attn_mfma(const void* qa, long ldq, void* out, long
               "latent_attn_mfma: the workspace is too small");
   const dim3 grid(n_splits == 0 ? ceil_div(tiles, 4) : (unsigned)tiles, n_splits == 0 ? 1 : n_splits);
   FMS_REQUIRE(tiles <= 0x7fffffffL && grid.y <= 65535, "latent_attn_mfma: too many tiles for one launch");
-#define LAUNCH_LATENT(RT, WC)                                                                                                  \
-  latent_attn_mfma_kernel<RT, WC><<<grid, 256, 0, stream>>>((const bf16*)qa, ldq, (bf16*)out, ldo, (float*)workspace, positions, \
-                                                            seq_of_token, block_table, table_stride, (const bf16*)cache,       \
-                                                            (const bf16*)vt_cache, sink, n_tokens, nheads, rank, width, scale, \
-                                                            window, tiles_per_token, n_parts)
-  if (rank <= 128 && width <= 192) LAUNCH_LATENT(8, 6);
-  else if (rank <= 256 && width <= 320) LAUNCH_LATENT(16, 10);
-  else LAUNCH_LATENT(32, 18);
+  // LDS: every wave's queries; for prompts also a tile of 32 key rows and the same keys' latent, transposed, which the
+  // waves of a block share
+#define LAUNCH_LATENT(RT, WC)                                                                                                      \
+  const size_t q_lds = (size_t)4 * WC * 64 * 8 * sizeof(bf16); /* the four waves' queries */                                       \
+  const size_t lds = q_lds + (size_t)(32 * (width + 8) + rank * 40) * sizeof(bf16);                                                \
+  static bool allowed = false; /* more than 64 KB of LDS a block has to be asked for, once a kernel */                             \
+  if (!allowed) {                                                                                                                  \
+    hipError_t e1 = hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<RT, WC, true>,                                        \
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                                   \
+    hipError_t e2 = hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<RT, WC, false>,                                       \
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                                   \
+    FMS_REQUIRE(e1 == hipSuccess && e2 == hipSuccess, "latent_attn_mfma: the kernel's LDS could not be sized: %s",                 \
+                hipGetErrorString(e1 != hipSuccess ? e1 : e2));                                                                    \
+    allowed = true;                                                                                                                \
+  }                                                                                                                                \
+  FMS_REQUIRE(lds <= 160 * 1024, "latent_attn_mfma: %zu bytes of LDS", lds);                                                       \
+  if (n_splits == 0)                                                                                                               \
+    latent_attn_mfma_kernel<RT, WC, true><<<grid, 256, lds, stream>>>((const bf16*)qa, ldq, (bf16*)out, ldo, (float*)workspace,   \
+                                                                      positions, seq_of_token, block_table, table_stride,         \
+                                                                      (const bf16*)cache, (const bf16*)vt_cache, sink, n_tokens,  \
+                                                                      nheads, rank, width, scale, window, tiles_per_token, n_parts); \
+  else                                                                                                                             \
+    latent_attn_mfma_kernel<RT, WC, false><<<grid, 256, q_lds, stream>>>((const bf16*)qa, ldq, (bf16*)out, ldo, (float*)workspace,    \
+                                                                     positions, seq_of_token, block_table, table_stride,          \
+                                                                     (const bf16*)cache, (const bf16*)vt_cache, sink, n_tokens,   \
+                                                                     nheads, rank, width, scale, window, tiles_per_token, n_parts)
+  if (rank <= 128 && width <= 192) {
+    LAUNCH_LATENT(8, 6);
+  } else if (rank <= 256 && width <= 320) {
+    LAUNCH_LATENT(16, 10);
+  } else {
+    LAUNCH_LATENT(32, 18);
+  }
 #undef LAUNCH_LATENT
   FMS_LAUNCH_CHECK("latent_attn_mfma");
   if (n_parts > 1) {

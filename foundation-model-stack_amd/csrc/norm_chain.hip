@@ -45,6 +45,53 @@ __global__ void __launch_bounds__(256)
   for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = from_f32<T>(row[i] * rs * load_scale(w, w_dtype, i));
 }
 
+// The same for rows of at most 256 * KEEP elements: branch, stream and both weights are asked for at once and wait in
+// registers, so the kernel pays the memory's latency once instead of four times (a decode step's rows are few, and
+// nothing else hides it).  The loops over what is kept have compile-time trip counts.
+template <typename T, int KEEP>
+__global__ void __launch_bounds__(256)
+    norm_add_norm_small_kernel(float* __restrict__ resid, const T* __restrict__ branch, const void* __restrict__ wb, float eps_b,
+                               const void* __restrict__ w, int w_dtype, float eps, T* __restrict__ out,
+                               const int* __restrict__ rows, int width) {
+  __shared__ float scratch[17];
+  const int r = rows ? rows[blockIdx.x] : blockIdx.x;
+  float* x = resid + (size_t)r * width;
+  const T* b = branch + (size_t)r * width;
+  float bv[KEEP], xv[KEEP], wbv[KEEP], wv[KEEP];
+  float sq = 0.f;
+#pragma unroll
+  for (int n = 0; n < KEEP; ++n) {
+    const int i = threadIdx.x + n * 256;
+    bv[n] = 0.f, xv[n] = 0.f, wbv[n] = 1.f, wv[n] = 1.f;
+    if (i < width) {
+      bv[n] = to_f32(b[i]);
+      xv[n] = x[i];
+      wbv[n] = load_scale(wb, w_dtype, i);
+      wv[n] = load_scale(w, w_dtype, i);
+    }
+    sq = fmaf(bv[n], bv[n], sq);
+  }
+  const float rb = rsqrtf(block_sum(sq, scratch) / (float)width + eps_b);
+  sq = 0.f;
+#pragma unroll
+  for (int n = 0; n < KEEP; ++n) {
+    const int i = threadIdx.x + n * 256;
+    xv[n] = xv[n] + bv[n] * rb * wbv[n];
+    if (i < width) {
+      if (!rows) x[i] = xv[n];
+      sq = fmaf(xv[n], xv[n], sq);
+    }
+  }
+  if (out == nullptr) return;
+  const float rs = rsqrtf(block_sum(sq, scratch) / (float)width + eps);
+  T* o = out + (size_t)blockIdx.x * width;
+#pragma unroll
+  for (int n = 0; n < KEEP; ++n) {
+    const int i = threadIdx.x + n * 256;
+    if (i < width) o[i] = from_f32<T>(xv[n] * rs * wv[n]);
+  }
+}
+
 extern "C" int fmsamd_norm_add_norm(float* resid, const void* branch, int act_dtype, const void* branch_weight,
                                     float branch_eps, const void* weight, int weight_dtype, float eps, void* out,
                                     const int* rows, int n_out, int width, hipStream_t stream) {
@@ -52,6 +99,16 @@ extern "C" int fmsamd_norm_add_norm(float* resid, const void* branch, int act_dt
   FMS_REQUIRE(n_out > 0 && width > 0 && width <= 16384, "norm_add_norm: bad sizes rows=%d width=%d", n_out, width);
   FMS_REQUIRE(resid != nullptr && branch != nullptr, "norm_add_norm: the stream and the branch are needed");
   const size_t lds = (size_t)width * sizeof(float);
+  if (width <= 256 * 8 && (act_dtype == FMS_F32 || act_dtype == FMS_BF16)) {
+    if (act_dtype == FMS_F32)
+      norm_add_norm_small_kernel<float, 8><<<n_out, 256, 0, stream>>>(resid, (const float*)branch, branch_weight, branch_eps, weight,
+                                                                       weight_dtype, eps, (float*)out, rows, width);
+    else
+      norm_add_norm_small_kernel<bf16, 8><<<n_out, 256, 0, stream>>>(resid, (const bf16*)branch, branch_weight, branch_eps, weight,
+                                                                      weight_dtype, eps, (bf16*)out, rows, width);
+    FMS_LAUNCH_CHECK("norm_add_norm");
+    return 0;
+  }
   if (act_dtype == FMS_F32)
     norm_add_norm_kernel<float><<<n_out, 256, lds, stream>>>(resid, (const float*)branch, branch_weight, branch_eps,
                                                              weight, weight_dtype, eps, (float*)out, rows, width);

@@ -3,10 +3,11 @@
 //
 //   tile_product_fma:  256 threads, 16 rows x 64 columns, any element type, any K, float32 FMA (the true 32-bit
 //                      path, and the path for rows that are not 16-byte aligned).
-//   tile_product_mfma: 256 threads = 4 waves, 16 rows x 256 columns (a wave: 64 columns as four 16x16 tiles),
+//   tile_product_mfma: 256 threads = 4 waves, 16 rows x 128 columns (a wave: 32 columns as two 16x16 tiles),
 //                      bfloat16 operands loaded straight from global memory into the operand layout of the
 //                      16x16x32 matrix instruction (a lane holds 8 consecutive k of one row); K a multiple of 8
-//                      and rows aligned to 16 bytes.
+//                      and rows aligned to 16 bytes.  The weights stream through once: four steps of K are asked
+//                      for before the first is multiplied, so that a wave keeps a dozen loads in flight.
 //
 // a_row(m), m < 16, and w_row(n) return the row's first element or nullptr for a row that is not there (zeros).
 #pragma once
@@ -15,7 +16,8 @@
 
 #define TILE_ROWS 16
 #define TILE_FMA_COLS 64
-#define TILE_MFMA_COLS 256
+#define TILE_MFMA_COLS 128
+#define TILE_MFMA_WAVE_TILES 2  // 16-column tiles a wave
 #define TILE_THREADS 256
 
 // After the call, thread tid holds acc[i] = C[row (tid / 64) * 4 + i][column tid % 64].
@@ -52,28 +54,35 @@ __device__ __forceinline__ void tile_product_fma(ARow a_row, WRow w_row, int K, 
   }
 }
 
-// After the call, lane l of wave w holds acc[t][i] = C[row (l / 16) * 4 + i][column w * 64 + t * 16 + l % 16].
-// w_row(n) takes n < 256, the column inside the block's tile.
+// After the call, lane l of wave w holds acc[t][i] = C[row (l / 16) * 4 + i][column w * 32 + t * 16 + l % 16].
+// w_row(n) takes n < 128, the column inside the block's tile.
 template <typename ARow, typename WRow>
-__device__ __forceinline__ void tile_product_mfma(ARow a_row, WRow w_row, int K, f32x4 (&acc)[4]) {
+__device__ __forceinline__ void tile_product_mfma(ARow a_row, WRow w_row, int K, f32x4 (&acc)[TILE_MFMA_WAVE_TILES]) {
+  constexpr int NT = TILE_MFMA_WAVE_TILES, AHEAD = 4;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, kq = (lane >> 4) * 8;
   const bf16* a = a_row(r);
-  const bf16* w[4];
+  const bf16* w[NT];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    w[t] = w_row(wave * 64 + t * 16 + r);
+  for (int t = 0; t < NT; ++t) {
+    w[t] = w_row(wave * (16 * NT) + t * 16 + r);
     acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  for (int k0 = 0; k0 < K; k0 += 32) {
-    const int k = k0 + kq;
-    const bool in = k < K;
-    const bf16x8 av = (in && a) ? *reinterpret_cast<const bf16x8*>(a + k) : zero;
+  for (int k0 = 0; k0 < K; k0 += 32 * AHEAD) {
+    bf16x8 av[AHEAD], wv[AHEAD][NT];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const bf16x8 wv = (in && w[t]) ? *reinterpret_cast<const bf16x8*>(w[t] + k) : zero;
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, wv, acc[t], 0, 0, 0);
+    for (int s = 0; s < AHEAD; ++s) {
+      const int k = k0 + 32 * s + kq;
+      const bool in = k < K;
+      av[s] = (in && a) ? *reinterpret_cast<const bf16x8*>(a + k) : zero;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) wv[s][t] = (in && w[t]) ? *reinterpret_cast<const bf16x8*>(w[t] + k) : zero;
+    }
+#pragma unroll
+    for (int s = 0; s < AHEAD; ++s) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[s], wv[s][t], acc[t], 0, 0, 0);
     }
   }
 }

@@ -690,10 +690,11 @@ def latent_attention_fits_mfma(rank: int, rot: int) -> bool:
 
 
 def latent_attention_splits(n_tokens: int, nheads: int, max_context: int) -> int:
-    """How many blocks share one (token, 16 heads) of the decode step of the MFMA kernel: enough for a few hundred
-    blocks in all, and no block with fewer than four tiles of 32 keys (one for each of its waves)."""
+    """How many blocks share one (token, 16 heads) of the decode step of the MFMA kernel: enough for some 256 blocks in
+    all (one a compute unit), no wave with fewer than four tiles of 32 keys at the context bound, at most 32 (every
+    part's result goes through the workspace and is merged)."""
     tiles = n_tokens * -(-nheads // 16)
-    return max(1, min(-(-512 // tiles), -(-max_context // 32) // 4, 64))
+    return max(1, min(-(-256 // tiles), -(-max_context // 32) // 16, 32))
 
 
 def _check_tables(cos, sin, rot: int) -> int:
