@@ -77,7 +77,7 @@ extern "C" int fmsamd_moe_route(const float* logits, long ld, int n_tokens, int 
 // --------------------------------------------------------------------------
 __global__ void __launch_bounds__(1024)
     group_kernel(const int* __restrict__ ids, int n_pairs, int n_experts, int* __restrict__ order, int* __restrict__ tiles,
-                 int max_tiles) {
+                 int max_tiles, int tile_rows) {
   __shared__ int counts[ROUTE_MAX_EXPERTS];
   __shared__ int cursor[ROUTE_MAX_EXPERTS];
   for (int e = threadIdx.x; e < n_experts; e += blockDim.x) counts[e] = 0;
@@ -92,10 +92,10 @@ __global__ void __launch_bounds__(1024)
     for (int e = 0; e < n_experts; ++e) {
       cursor[e] = at;
       const int c = counts[e];
-      for (int r = 0; r < c && nt < max_tiles; r += TILE_ROWS, ++nt) {
+      for (int r = 0; r < c && nt < max_tiles; r += tile_rows, ++nt) {
         tiles[3 * nt] = e;
         tiles[3 * nt + 1] = at + r;
-        tiles[3 * nt + 2] = c - r < TILE_ROWS ? c - r : TILE_ROWS;
+        tiles[3 * nt + 2] = c - r < tile_rows ? c - r : tile_rows;
       }
       at += c;
     }
@@ -108,18 +108,26 @@ __global__ void __launch_bounds__(1024)
   }
 }
 
-extern "C" int fmsamd_moe_max_tiles(int n_pairs, int n_experts) {
-  return (n_pairs + TILE_ROWS - 1) / TILE_ROWS + (n_experts < n_pairs ? n_experts : n_pairs);
+// Rows of a tile: 64 where the experts have that many rows on average (prompts) and the matrix-core kernel can run
+// (wide_ok: bfloat16, rows aligned to 16 bytes), else 16.
+extern "C" int fmsamd_moe_tile_rows(int n_pairs, int n_experts, int wide_ok) {
+  return (wide_ok && n_pairs >= (long)TILE_WIDE_ROWS * n_experts) ? TILE_WIDE_ROWS : TILE_ROWS;
+}
+
+extern "C" int fmsamd_moe_max_tiles(int n_pairs, int n_experts, int tile_rows) {
+  if (tile_rows <= 0) return 0;
+  return (n_pairs + tile_rows - 1) / tile_rows + (n_experts < n_pairs ? n_experts : n_pairs);
 }
 
 extern "C" int fmsamd_moe_group(const int* ids, int n_pairs, int n_experts, int* order, int* tiles, int max_tiles,
-                                hipStream_t stream) {
+                                int tile_rows, hipStream_t stream) {
   if (n_pairs == 0) return 0;
   FMS_REQUIRE(n_pairs > 0 && n_experts > 0 && n_experts <= ROUTE_MAX_EXPERTS, "moe_group: %d pairs, %d experts (at most %d)", n_pairs,
               n_experts, ROUTE_MAX_EXPERTS);
-  FMS_REQUIRE(max_tiles >= fmsamd_moe_max_tiles(n_pairs, n_experts), "moe_group: room for %d tiles, %d may be needed", max_tiles,
-              fmsamd_moe_max_tiles(n_pairs, n_experts));
-  group_kernel<<<1, 1024, 0, stream>>>(ids, n_pairs, n_experts, order, tiles, max_tiles);
+  FMS_REQUIRE(tile_rows == TILE_ROWS || tile_rows == TILE_WIDE_ROWS, "moe_group: tiles of %d rows", tile_rows);
+  FMS_REQUIRE(max_tiles >= fmsamd_moe_max_tiles(n_pairs, n_experts, tile_rows), "moe_group: room for %d tiles, %d may be needed", max_tiles,
+              fmsamd_moe_max_tiles(n_pairs, n_experts, tile_rows));
+  group_kernel<<<1, 1024, 0, stream>>>(ids, n_pairs, n_experts, order, tiles, max_tiles, tile_rows);
   FMS_LAUNCH_CHECK("moe_group");
   return 0;
 }
@@ -232,12 +240,68 @@ __global__ void __launch_bounds__(TILE_THREADS) expert_down_mfma_kernel(ExpertAr
   }
 }
 
+// The same two products on tiles of 64 rows (tile_product_mfma_wide).
+__global__ void __launch_bounds__(TILE_THREADS) expert_gate_up_wide_kernel(ExpertArgs a) {
+  const int e = a.tiles[3 * blockIdx.x], start = a.tiles[3 * blockIdx.x + 1], rows = a.tiles[3 * blockIdx.x + 2];
+  if (rows == 0) return;
+  const int n0 = blockIdx.y * TILE_MFMA_COLS;
+  const bf16* x = (const bf16*)a.x;
+  const bf16* wg = (const bf16*)a.w1 + (size_t)e * a.N * a.K;
+  const bf16* wu = (const bf16*)a.w2 + (size_t)e * a.N * a.K;
+  auto a_row = [&](int m) { return m < rows ? x + (size_t)(a.order[start + m] / a.top) * a.ldx : (const bf16*)nullptr; };
+  f32x4 g[2][4], u[2][4];
+  tile_product_mfma_wide(a_row, [&](int n) { return n0 + n < a.N ? wg + (size_t)(n0 + n) * a.K : (const bf16*)nullptr; }, a.K, g);
+  tile_product_mfma_wide(a_row, [&](int n) { return n0 + n < a.N ? wu + (size_t)(n0 + n) * a.K : (const bf16*)nullptr; }, a.K, u);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = (wave >> 1) * 32 + mt * 16 + (lane >> 4) * 4 + i;
+      if (m >= rows) continue;
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) {
+        const int n = n0 + (wave & 1) * 64 + nt * 16 + (lane & 15);
+        if (n < a.N) ((bf16*)a.y)[(size_t)(start + m) * a.N + n] = (bf16)clamp_gated(g[mt][nt][i], u[mt][nt][i], a.limit, a.alpha, a.shift);
+      }
+    }
+  }
+}
+
+__global__ void __launch_bounds__(TILE_THREADS) expert_down_wide_kernel(ExpertArgs a) {
+  const int e = a.tiles[3 * blockIdx.x], start = a.tiles[3 * blockIdx.x + 1], rows = a.tiles[3 * blockIdx.x + 2];
+  if (rows == 0) return;
+  const int n0 = blockIdx.y * TILE_MFMA_COLS;
+  const bf16* x = (const bf16*)a.x;
+  const bf16* w = (const bf16*)a.w1 + (size_t)e * a.N * a.K;
+  f32x4 acc[2][4];
+  tile_product_mfma_wide([&](int m) { return m < rows ? x + (size_t)(start + m) * a.ldx : (const bf16*)nullptr; },
+                         [&](int n) { return n0 + n < a.N ? w + (size_t)(n0 + n) * a.K : (const bf16*)nullptr; }, a.K, acc);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = (wave >> 1) * 32 + mt * 16 + (lane >> 4) * 4 + i;
+      if (m >= rows) continue;
+      float* yrow = (float*)a.y + (size_t)a.order[start + m] * a.N;
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) {
+        const int n = n0 + (wave & 1) * 64 + nt * 16 + (lane & 15);
+        if (n < a.N) yrow[n] = acc[mt][nt][i];
+      }
+    }
+  }
+}
+
 // stage 0: hidden = act(x Wg^T, x Wu^T) for the tiles' rows; stage 1: y = hidden Wd^T
+// tile_rows: what fmsamd_moe_tile_rows said when the tiles were made
 extern "C" int fmsamd_moe_experts(int stage, const void* x, long ldx, const void* w1, const void* w2, void* y, int dtype,
-                                  const int* order, const int* tiles, int max_tiles, int top, int N, int K, float limit,
-                                  float alpha, float shift, hipStream_t stream) {
+                                  const int* order, const int* tiles, int max_tiles, int tile_rows, int top, int N, int K,
+                                  float limit, float alpha, float shift, hipStream_t stream) {
   if (max_tiles == 0) return 0;
   FMS_REQUIRE(stage == 0 || stage == 1, "moe_experts: stage %d", stage);
+  FMS_REQUIRE(tile_rows == TILE_ROWS || tile_rows == TILE_WIDE_ROWS, "moe_experts: tiles of %d rows", tile_rows);
   FMS_REQUIRE(max_tiles > 0 && top > 0 && N > 0 && K > 0 && ldx >= K, "moe_experts: bad sizes tiles=%d top=%d N=%d K=%d ldx=%ld", max_tiles,
               top, N, K, ldx);
   ExpertArgs a{x, ldx, w1, w2, y, order, tiles, top, N, K, limit, alpha, shift};
@@ -245,7 +309,12 @@ extern "C" int fmsamd_moe_experts(int stage, const void* x, long ldx, const void
                     (w2 == nullptr || ((uintptr_t)w2 % 16) == 0);
   const dim3 grid(max_tiles, ceil_div(N, mfma ? TILE_MFMA_COLS : TILE_FMA_COLS));
   FMS_REQUIRE(grid.y <= 65535, "moe_experts: %d columns are too many for one launch", N);
-  if (dtype == FMS_F32) {
+  if (tile_rows == TILE_WIDE_ROWS) {
+    // tiles of 64 rows are made for the matrix-core kernel only
+    FMS_REQUIRE(mfma, "moe_experts: tiles of %d rows need bfloat16 rows aligned to 16 bytes", tile_rows);
+    if (stage == 0) expert_gate_up_wide_kernel<<<grid, TILE_THREADS, 0, stream>>>(a);
+    else expert_down_wide_kernel<<<grid, TILE_THREADS, 0, stream>>>(a);
+  } else if (dtype == FMS_F32) {
     if (stage == 0) expert_gate_up_fma_kernel<float><<<grid, TILE_THREADS, 0, stream>>>(a);
     else expert_down_fma_kernel<float><<<grid, TILE_THREADS, 0, stream>>>(a);
   } else if (dtype == FMS_BF16) {

@@ -218,12 +218,17 @@ int fmsamd_latent_attn_mfma(const void* qa, long ldq, void* out, long ldo, void*
 // ---- experts (experts.hip) -----------------------------------------------------------------------------------------
 int fmsamd_moe_route(const float* logits, long ld, int n_tokens, int n_experts, int top, int* ids, float* weights,
                      hipStream_t stream);
-int fmsamd_moe_max_tiles(int n_pairs, int n_experts);
-// order [n_pairs], tiles [max_tiles][3] = (expert, first row in order, rows)
-int fmsamd_moe_group(const int* ids, int n_pairs, int n_experts, int* order, int* tiles, int max_tiles, hipStream_t stream);
+// Rows of a tile of (token, choice) pairs of one expert: 64 where experts have many rows and the matrix-core kernel can
+// run (wide_ok), else 16; the most tiles there can be; the pairs sorted by expert and cut into tiles:
+// order [n_pairs], tiles [max_tiles][3] = (expert, first row in order, rows).
+int fmsamd_moe_tile_rows(int n_pairs, int n_experts, int wide_ok);
+int fmsamd_moe_max_tiles(int n_pairs, int n_experts, int tile_rows);
+int fmsamd_moe_group(const int* ids, int n_pairs, int n_experts, int* order, int* tiles, int max_tiles, int tile_rows,
+                     hipStream_t stream);
+// stage 0: y[sorted pair] = act(x Wg^T, x Wu^T) (w1, w2 = gate, up [E, N, K]); stage 1: y[pair] = x W^T, float32
 int fmsamd_moe_experts(int stage, const void* x, long ldx, const void* w1, const void* w2, void* y, int dtype,
-                       const int* order, const int* tiles, int max_tiles, int top, int N, int K, float limit, float alpha,
-                       float shift, hipStream_t stream);
+                       const int* order, const int* tiles, int max_tiles, int tile_rows, int top, int N, int K, float limit,
+                       float alpha, float shift, hipStream_t stream);
 int fmsamd_moe_combine(const float* y, const float* weights, int top, const void* shared, const float* shared_gate, long ldg,
                        void* out, int dtype, int n_tokens, int width, hipStream_t stream);
 

@@ -334,11 +334,9 @@ struct LatentState {
   float m, l;
 };
 
-template <int RT, int WC, typename LoadQ, typename LoadK, typename LoadV>
+template <int RT, int WC, int KG, int VG, typename LoadQ, typename LoadK, typename LoadV>
 __device__ __forceinline__ void latent_tile(LatentState<RT, WC>& st, LoadQ load_q, LoadK load_k, LoadV load_v, int base,
                                             int lo, int pos, int rank, int width, float scale, int grp) {
-  constexpr int KG = WC <= 10 ? WC : 6;
-  constexpr int VG = RT <= 16 ? RT : 8;
   f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int c0 = 0; c0 < WC; c0 += KG) {
@@ -380,6 +378,9 @@ __device__ __forceinline__ void latent_tile(LatentState<RT, WC>& st, LoadQ load_
   }
   st.l = st.l * alpha + psum;
   st.m = m_new;
+  // Once a column's maximum has settled, alpha is one: the accumulators (which live in the matrix unit's registers
+  // and have to be moved out and back to be scaled) are left alone unless some column's maximum rose.
+  const bool rescale = __any(alpha != 1.f);
 #pragma unroll
   for (int d0 = 0; d0 < RT; d0 += VG) {
     bf16x8 v[VG];
@@ -390,8 +391,10 @@ __device__ __forceinline__ void latent_tile(LatentState<RT, WC>& st, LoadQ load_
 #pragma unroll
     for (int dt = 0; dt < VG; ++dt) {
       if (d0 + dt < RT && (d0 + dt) * 16 < rank) {
+        if (rescale) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) st.acc[d0 + dt][i] *= alpha;
+          for (int i = 0; i < 4; ++i) st.acc[d0 + dt][i] *= alpha;
+        }
         st.acc[d0 + dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v[dt], pmat, st.acc[d0 + dt], 0, 0, 0);
       }
     }
@@ -523,24 +526,44 @@ __global__ void __launch_bounds__(256)
     }
     const int* bt = block_table + (size_t)any_seq * table_stride;
     const int chunks_k = width / 8;  // 16-byte pieces in a key row
-    for (int base = (first_lo / 32) * 32; base <= last_pos; base += 32) {
+    // A thread's pieces of a tile: KP 16-byte pieces of the key rows, VP of the transposed latent.  The next tile's
+    // pieces are asked for before this tile is worked on and wait in registers until every wave is done with it.
+    constexpr int KP = (32 * WC * 4 + 255) / 256, VP = (RT * 16 * 4 + 255) / 256;
+    bf16x8 kpre[KP], vpre[VP];
+    auto fetch = [&](int base) {
       const size_t page = readable_page(uniform_load(bt + base / PAGE_TOKENS));
       const int in_page = base % PAGE_TOKENS;
-      __syncthreads();  // the tile before this one has been read by every wave
-      for (int i = threadIdx.x; i < 32 * chunks_k; i += 256) {
-        const int r = i / chunks_k, ch = i % chunks_k;
-        *reinterpret_cast<bf16x8*>(k_lds + r * ks + ch * 8) =
-            *reinterpret_cast<const bf16x8*>(cache + (page * PAGE_TOKENS + in_page + r) * width + ch * 8);
+#pragma unroll
+      for (int n = 0; n < KP; ++n) {
+        const int i = threadIdx.x + n * 256;
+        if (i < 32 * chunks_k)
+          kpre[n] = *reinterpret_cast<const bf16x8*>(cache + (page * PAGE_TOKENS + in_page + i / chunks_k) * width + (i % chunks_k) * 8);
       }
-      for (int i = threadIdx.x; i < rank * 4; i += 256) {
-        const int d = i >> 2, ch = i & 3;
-        *reinterpret_cast<bf16x8*>(v_lds + d * vs + ch * 8) =
-            *reinterpret_cast<const bf16x8*>(vt_cache + (page * rank + d) * PAGE_TOKENS + in_page + ch * 8);
+#pragma unroll
+      for (int n = 0; n < VP; ++n) {
+        const int i = threadIdx.x + n * 256;
+        if (i < rank * 4) vpre[n] = *reinterpret_cast<const bf16x8*>(vt_cache + (page * rank + (i >> 2)) * PAGE_TOKENS + in_page + (i & 3) * 8);
+      }
+    };
+    const int first_base = (first_lo / 32) * 32;
+    if (first_base <= last_pos) fetch(first_base);
+    for (int base = first_base; base <= last_pos; base += 32) {
+      __syncthreads();  // the tile before this one has been read by every wave
+#pragma unroll
+      for (int n = 0; n < KP; ++n) {
+        const int i = threadIdx.x + n * 256;
+        if (i < 32 * chunks_k) *reinterpret_cast<bf16x8*>(k_lds + (i / chunks_k) * ks + (i % chunks_k) * 8) = kpre[n];
+      }
+#pragma unroll
+      for (int n = 0; n < VP; ++n) {
+        const int i = threadIdx.x + n * 256;
+        if (i < rank * 4) *reinterpret_cast<bf16x8*>(v_lds + (i >> 2) * vs + (i & 3) * 8) = vpre[n];
       }
       __syncthreads();
+      if (base + 32 <= last_pos) fetch(base + 32);
       // (a condition that all lanes of the wave share: matrix instructions take their operands from every lane)
       if (tile < n_tiles && seq >= 0 && base <= pos) {
-        latent_tile<RT, WC>(
+        latent_tile<RT, WC, (WC <= 10 ? WC : 6), (RT <= 16 ? RT : 8)>(
             st, load_q,
             [&](int which, int c) {
               return c * 32 + grp * 8 < width ? *reinterpret_cast<const bf16x8*>(k_lds + (key_a + 4 * which) * ks + c * 32 + grp * 8) : zero8;
@@ -564,7 +587,8 @@ __global__ void __launch_bounds__(256)
       const int in_page = base % PAGE_TOKENS;
       const bf16* ka = cache + (page * PAGE_TOKENS + in_page + key_a) * width + grp * 8;
       const bf16* vt = vt_cache + (page * rank + col) * PAGE_TOKENS + in_page + grp * 8;
-      latent_tile<RT, WC>(
+      // straight from global memory: half a tile of key loads, then half its latent loads, in flight at once (all of them up to medium sizes)
+      latent_tile<RT, WC, (WC <= 10 ? WC : 9), (RT <= 16 ? RT : 16)>(
           st, load_q,
           [&](int which, int c) {
             return c * 32 + grp * 8 < width ? *reinterpret_cast<const bf16x8*>(ka + which * 4 * (size_t)width + c * 32) : zero8;

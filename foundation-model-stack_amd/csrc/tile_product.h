@@ -9,7 +9,11 @@
 //                      and rows aligned to 16 bytes.  The weights stream through once: four steps of K are asked
 //                      for before the first is multiplied, so that a wave keeps a dozen loads in flight.
 //
-// a_row(m), m < 16, and w_row(n) return the row's first element or nullptr for a row that is not there (zeros).
+//   tile_product_mfma_wide: the same for 64 rows x 128 columns, a wave 32 rows x 64 columns (2 x 4 tiles): eight
+//                      products for six loads instead of two for three, for steps of many rows (prompts), whose
+//                      products are bound by what the caches deliver.
+//
+// a_row(m), m < 16 (64 for the wide tile), and w_row(n) return the row's first element or nullptr for a row that is not there (zeros).
 #pragma once
 
 #include "common.h"
@@ -83,6 +87,48 @@ __device__ __forceinline__ void tile_product_mfma(ARow a_row, WRow w_row, int K,
     for (int s = 0; s < AHEAD; ++s) {
 #pragma unroll
       for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[s], wv[s][t], acc[t], 0, 0, 0);
+    }
+  }
+}
+
+#define TILE_WIDE_ROWS 64
+// After the call, lane l of wave w holds
+//   acc[mt][nt][i] = C[row (w / 2) * 32 + mt * 16 + (l / 16) * 4 + i][column (w % 2) * 64 + nt * 16 + l % 16].
+template <typename ARow, typename WRow>
+__device__ __forceinline__ void tile_product_mfma_wide(ARow a_row, WRow w_row, int K, f32x4 (&acc)[2][4]) {
+  constexpr int AHEAD = 2;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, kq = (lane >> 4) * 8;
+  const bf16* a[2];
+  const bf16* w[4];
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt) a[mt] = a_row((wave >> 1) * 32 + mt * 16 + r);
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) w[nt] = w_row((wave & 1) * 64 + nt * 16 + r);
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt) {
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int k0 = 0; k0 < K; k0 += 32 * AHEAD) {
+    bf16x8 av[AHEAD][2], wv[AHEAD][4];
+#pragma unroll
+    for (int s = 0; s < AHEAD; ++s) {
+      const int k = k0 + 32 * s + kq;
+      const bool in = k < K;
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) av[s][mt] = (in && a[mt]) ? *reinterpret_cast<const bf16x8*>(a[mt] + k) : zero;
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) wv[s][nt] = (in && w[nt]) ? *reinterpret_cast<const bf16x8*>(w[nt] + k) : zero;
+    }
+#pragma unroll
+    for (int s = 0; s < AHEAD; ++s) {
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) {
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[s][mt], wv[s][nt], acc[mt][nt], 0, 0, 0);
+      }
     }
   }
 }

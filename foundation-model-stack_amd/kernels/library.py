@@ -57,8 +57,8 @@ _SIGNATURES = {
     "fmsamd_headwise_linear": [P, L, L, P, P, L, L, P, L, I, I, I, I, I, P],
     "fmsamd_latent_attn_generic": [P, L, P, L, I, P, P, P, I, P, P, I, I, I, I, F, I, P],
     "fmsamd_moe_route": [P, L, I, I, I, P, P, P],
-    "fmsamd_moe_group": [P, I, I, P, P, I, P],
-    "fmsamd_moe_experts": [I, P, L, P, P, P, I, P, P, I, I, I, I, F, F, F, P],
+    "fmsamd_moe_group": [P, I, I, P, P, I, I, P],
+    "fmsamd_moe_experts": [I, P, L, P, P, P, I, P, P, I, I, I, I, I, F, F, F, P],
     "fmsamd_moe_combine": [P, P, I, P, P, L, P, I, I, I, P],
     "fmsamd_probe_read": [P, L, I, I, P, P],
     "fmsamd_probe_mfma": [I, I, I, P, P, P],
@@ -104,7 +104,9 @@ def load(verbose: bool = True) -> ctypes.CDLL:
         lib.fmsamd_latent_attn_mfma_fits.restype = c_int
         lib.fmsamd_latent_attn_mfma_fits.argtypes = [I, I]
         lib.fmsamd_moe_max_tiles.restype = c_int
-        lib.fmsamd_moe_max_tiles.argtypes = [I, I]
+        lib.fmsamd_moe_max_tiles.argtypes = [I, I, I]
+        lib.fmsamd_moe_tile_rows.restype = c_int
+        lib.fmsamd_moe_tile_rows.argtypes = [I, I, I]
         lib.fmsamd_argmax_workspace.restype = c_long
         lib.fmsamd_argmax_workspace.argtypes = [I, I]
         lib.fmsamd_attn_decode_workspace.restype = c_long

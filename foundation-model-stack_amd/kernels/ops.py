@@ -691,10 +691,10 @@ def latent_attention_fits_mfma(rank: int, rot: int) -> bool:
 
 def latent_attention_splits(n_tokens: int, nheads: int, max_context: int) -> int:
     """How many blocks share one (token, 16 heads) of the decode step of the MFMA kernel: enough for some 256 blocks in
-    all (one a compute unit), no wave with fewer than four tiles of 32 keys at the context bound, at most 32 (every
+    all (one a compute unit), no wave with fewer than two tiles of 32 keys at the context bound, at most 32 (every
     part's result goes through the workspace and is merged)."""
     tiles = n_tokens * -(-nheads // 16)
-    return max(1, min(-(-256 // tiles), -(-max_context // 32) // 16, 32))
+    return max(1, min(-(-256 // tiles), -(-max_context // 32) // 8, 32))
 
 
 def _check_tables(cos, sin, rot: int) -> int:
@@ -842,17 +842,20 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, gate_w: torch.Tensor, up_w: 
             raise TypeError("the experts' weights are contiguous and of the type of x")
     lib = load()
     n_pairs = T * top
-    max_tiles = lib.fmsamd_moe_max_tiles(n_pairs, E)
+    # tiles of 64 rows where the experts have many rows (prompts) and the matrix-core kernel can load the rows
+    wide_ok = x.dtype == torch.bfloat16 and width % 8 == 0 and ff % 8 == 0 and x.stride(0) % 8 == 0
+    tile_rows = lib.fmsamd_moe_tile_rows(n_pairs, E, int(wide_ok))
+    max_tiles = lib.fmsamd_moe_max_tiles(n_pairs, E, tile_rows)
     order = torch.empty(n_pairs, dtype=torch.int32, device=x.device)
     tiles = torch.empty(max_tiles, 3, dtype=torch.int32, device=x.device)
-    check(lib.fmsamd_moe_group(ids.data_ptr(), n_pairs, E, order.data_ptr(), tiles.data_ptr(), max_tiles, _stream()))
+    check(lib.fmsamd_moe_group(ids.data_ptr(), n_pairs, E, order.data_ptr(), tiles.data_ptr(), max_tiles, tile_rows, _stream()))
     hidden = torch.empty(n_pairs, ff, dtype=x.dtype, device=x.device)
     y = torch.empty(n_pairs, width, dtype=torch.float32, device=x.device)
     code = _code(x.dtype)
     check(lib.fmsamd_moe_experts(0, x.data_ptr(), x.stride(0), gate_w.data_ptr(), up_w.data_ptr(), hidden.data_ptr(), code,
-                                 order.data_ptr(), tiles.data_ptr(), max_tiles, top, ff, width, float(limit), float(alpha), float(shift), _stream()))
+                                 order.data_ptr(), tiles.data_ptr(), max_tiles, tile_rows, top, ff, width, float(limit), float(alpha), float(shift), _stream()))
     check(lib.fmsamd_moe_experts(1, hidden.data_ptr(), hidden.stride(0), down_w.data_ptr(), None, y.data_ptr(), code,
-                                 order.data_ptr(), tiles.data_ptr(), max_tiles, top, width, ff, float(limit), float(alpha), float(shift), _stream()))
+                                 order.data_ptr(), tiles.data_ptr(), max_tiles, tile_rows, top, width, ff, float(limit), float(alpha), float(shift), _stream()))
     return y
 
 

@@ -329,7 +329,7 @@ def test_router(lib, sizes):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("sizes", [(6, 2, 48, 128, 50), (5, 1, 36, 100, 7), (8, 8, 128, 256, 40), (3, 2, 20, 64, 1)])
+@pytest.mark.parametrize("sizes", [(6, 2, 48, 128, 50), (5, 1, 36, 100, 7), (8, 8, 128, 256, 40), (3, 2, 20, 64, 1), (4, 2, 64, 128, 300), (3, 3, 200, 72, 150)])
 def test_experts_and_their_sum(lib, dtype, sizes):
     from fms_amd.kernels import ops
 
