@@ -334,7 +334,9 @@ struct LatentState {
   float m, l;
 };
 
-template <int RT, int WC, int KG, int VG, typename LoadQ, typename LoadK, typename LoadV>
+// EXACT: the latent has exactly RT * 16 elements and a row exactly WC * 32, so no product of the loops below has
+// to be asked whether it exists (each such question is a branch around a matrix instruction).
+template <int RT, int WC, int KG, int VG, bool EXACT, typename LoadQ, typename LoadK, typename LoadV>
 __device__ __forceinline__ void latent_tile(LatentState<RT, WC>& st, LoadQ load_q, LoadK load_k, LoadV load_v, int base,
                                             int lo, int pos, int rank, int width, float scale, int grp) {
   f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
@@ -343,11 +345,11 @@ __device__ __forceinline__ void latent_tile(LatentState<RT, WC>& st, LoadQ load_
     bf16x8 ka[KG], kb[KG];
 #pragma unroll
     for (int c = 0; c < KG; ++c) {
-      if (c0 + c < WC && (c0 + c) * 32 < width) ka[c] = load_k(0, c0 + c), kb[c] = load_k(1, c0 + c);
+      if (c0 + c < WC && (EXACT || (c0 + c) * 32 < width)) ka[c] = load_k(0, c0 + c), kb[c] = load_k(1, c0 + c);
     }
 #pragma unroll
     for (int c = 0; c < KG; ++c) {
-      if (c0 + c < WC && (c0 + c) * 32 < width) {
+      if (c0 + c < WC && (EXACT || (c0 + c) * 32 < width)) {
         const bf16x8 q = load_q(c0 + c);
         sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[c], q, sa, 0, 0, 0);
         sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb[c], q, sb, 0, 0, 0);
@@ -386,11 +388,11 @@ __device__ __forceinline__ void latent_tile(LatentState<RT, WC>& st, LoadQ load_
     bf16x8 v[VG];
 #pragma unroll
     for (int dt = 0; dt < VG; ++dt) {
-      if (d0 + dt < RT && (d0 + dt) * 16 < rank) v[dt] = load_v(d0 + dt);
+      if (d0 + dt < RT && (EXACT || (d0 + dt) * 16 < rank)) v[dt] = load_v(d0 + dt);
     }
 #pragma unroll
     for (int dt = 0; dt < VG; ++dt) {
-      if (d0 + dt < RT && (d0 + dt) * 16 < rank) {
+      if (d0 + dt < RT && (EXACT || (d0 + dt) * 16 < rank)) {
         if (rescale) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) st.acc[d0 + dt][i] *= alpha;
@@ -402,7 +404,7 @@ __device__ __forceinline__ void latent_tile(LatentState<RT, WC>& st, LoadQ load_
 }
 
 // What a wave leaves: the normalised result (one part) or its part's maximum, sum and unnormalised result.
-template <int RT, int WC>
+template <int RT, int WC, bool EXACT>
 __device__ __forceinline__ void latent_finish(LatentState<RT, WC>& st, bf16* __restrict__ out, long ldo, float* __restrict__ ws, int t,
                                               int head, int nheads, int rank, int n_parts, int part, int grp) {
   st.l += __shfl_xor(st.l, 16, WAVE);
@@ -414,7 +416,7 @@ __device__ __forceinline__ void latent_finish(LatentState<RT, WC>& st, bf16* __r
     bf16* o = out + (size_t)t * ldo + (size_t)head * rank;
 #pragma unroll
     for (int dt = 0; dt < RT; ++dt) {
-      if (dt * 16 < rank) {
+      if (EXACT || dt * 16 < rank) {
         bf16x4 r = {(bf16)(st.acc[dt][0] * inv), (bf16)(st.acc[dt][1] * inv), (bf16)(st.acc[dt][2] * inv), (bf16)(st.acc[dt][3] * inv)};
         *reinterpret_cast<bf16x4*>(o + dt * 16 + grp * 4) = r;
       }
@@ -424,7 +426,7 @@ __device__ __forceinline__ void latent_finish(LatentState<RT, WC>& st, bf16* __r
     if (grp == 0) w[0] = st.m, w[1] = st.l;
 #pragma unroll
     for (int dt = 0; dt < RT; ++dt) {
-      if (dt * 16 < rank) *reinterpret_cast<f32x4*>(w + 4 + dt * 16 + grp * 4) = st.acc[dt];
+      if (EXACT || dt * 16 < rank) *reinterpret_cast<f32x4*>(w + 4 + dt * 16 + grp * 4) = st.acc[dt];
     }
   }
 }
@@ -433,7 +435,7 @@ __device__ __forceinline__ void latent_finish(LatentState<RT, WC>& st, bf16* __r
 // one token) share every tile of keys through LDS, so a tile comes from the caches once a block instead of once a
 // wave; a block whose tiles lie in different sequences, and every block of a decode step, loads straight from
 // global memory.
-template <int RT, int WC, bool LDS>
+template <int RT, int WC, bool LDS, bool EXACT>
 __global__ void __launch_bounds__(256)
     latent_attn_mfma_kernel(const bf16* __restrict__ qa, long ldq, bf16* __restrict__ out, long ldo, float* __restrict__ ws,
                             const int* __restrict__ positions, const int* __restrict__ seq_of_token,
@@ -500,7 +502,7 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
     for (int c = 0; c < WC; ++c) {
       const int k = c * 32 + grp * 8;
-      *reinterpret_cast<bf16x8*>(q_lds + c * 64 * 8) = (valid && k < width) ? *reinterpret_cast<const bf16x8*>(qrow + k) : zero8;
+      *reinterpret_cast<bf16x8*>(q_lds + c * 64 * 8) = (valid && (EXACT || k < width)) ? *reinterpret_cast<const bf16x8*>(qrow + k) : zero8;
     }
   }
   auto load_q = [&](int c) { return *reinterpret_cast<const bf16x8*>(q_lds + c * 64 * 8); };
@@ -530,19 +532,35 @@ __global__ void __launch_bounds__(256)
     // pieces are asked for before this tile is worked on and wait in registers until every wave is done with it.
     constexpr int KP = (32 * WC * 4 + 255) / 256, VP = (RT * 16 * 4 + 255) / 256;
     bf16x8 kpre[KP], vpre[VP];
+    // where this thread's pieces lie in a tile of the cache and in LDS: the same for every tile (the divisions are
+    // done once; -1: this thread has no such piece)
+    int k_from[KP], k_to[KP], v_from[VP], v_to[VP];
+#pragma unroll
+    for (int n = 0; n < KP; ++n) {
+      const int i = threadIdx.x + n * 256;
+      const bool has = i < 32 * chunks_k;
+      k_from[n] = has ? (i / chunks_k) * width + (i % chunks_k) * 8 : -1;
+      k_to[n] = has ? (i / chunks_k) * ks + (i % chunks_k) * 8 : -1;
+    }
+#pragma unroll
+    for (int n = 0; n < VP; ++n) {
+      const int i = threadIdx.x + n * 256;
+      const bool has = i < rank * 4;
+      v_from[n] = has ? (i >> 2) * PAGE_TOKENS + (i & 3) * 8 : -1;
+      v_to[n] = has ? (i >> 2) * vs + (i & 3) * 8 : -1;
+    }
     auto fetch = [&](int base) {
       const size_t page = readable_page(uniform_load(bt + base / PAGE_TOKENS));
       const int in_page = base % PAGE_TOKENS;
+      const bf16* kp = cache + (page * PAGE_TOKENS + in_page) * width;
+      const bf16* vp = vt_cache + page * rank * PAGE_TOKENS + in_page;
 #pragma unroll
       for (int n = 0; n < KP; ++n) {
-        const int i = threadIdx.x + n * 256;
-        if (i < 32 * chunks_k)
-          kpre[n] = *reinterpret_cast<const bf16x8*>(cache + (page * PAGE_TOKENS + in_page + i / chunks_k) * width + (i % chunks_k) * 8);
+        if (k_from[n] >= 0) kpre[n] = *reinterpret_cast<const bf16x8*>(kp + k_from[n]);
       }
 #pragma unroll
       for (int n = 0; n < VP; ++n) {
-        const int i = threadIdx.x + n * 256;
-        if (i < rank * 4) vpre[n] = *reinterpret_cast<const bf16x8*>(vt_cache + (page * rank + (i >> 2)) * PAGE_TOKENS + in_page + (i & 3) * 8);
+        if (v_from[n] >= 0) vpre[n] = *reinterpret_cast<const bf16x8*>(vp + v_from[n]);
       }
     };
     const int first_base = (first_lo / 32) * 32;
@@ -551,22 +569,20 @@ __global__ void __launch_bounds__(256)
       __syncthreads();  // the tile before this one has been read by every wave
 #pragma unroll
       for (int n = 0; n < KP; ++n) {
-        const int i = threadIdx.x + n * 256;
-        if (i < 32 * chunks_k) *reinterpret_cast<bf16x8*>(k_lds + (i / chunks_k) * ks + (i % chunks_k) * 8) = kpre[n];
+        if (k_to[n] >= 0) *reinterpret_cast<bf16x8*>(k_lds + k_to[n]) = kpre[n];
       }
 #pragma unroll
       for (int n = 0; n < VP; ++n) {
-        const int i = threadIdx.x + n * 256;
-        if (i < rank * 4) *reinterpret_cast<bf16x8*>(v_lds + (i >> 2) * vs + (i & 3) * 8) = vpre[n];
+        if (v_to[n] >= 0) *reinterpret_cast<bf16x8*>(v_lds + v_to[n]) = vpre[n];
       }
       __syncthreads();
       if (base + 32 <= last_pos) fetch(base + 32);
       // (a condition that all lanes of the wave share: matrix instructions take their operands from every lane)
       if (tile < n_tiles && seq >= 0 && base <= pos) {
-        latent_tile<RT, WC, (WC <= 10 ? WC : 6), (RT <= 16 ? RT : 8)>(
+        latent_tile<RT, WC, (WC <= 10 ? WC : 6), (RT <= 16 ? RT : 8), EXACT>(
             st, load_q,
             [&](int which, int c) {
-              return c * 32 + grp * 8 < width ? *reinterpret_cast<const bf16x8*>(k_lds + (key_a + 4 * which) * ks + c * 32 + grp * 8) : zero8;
+              return (EXACT || c * 32 + grp * 8 < width) ? *reinterpret_cast<const bf16x8*>(k_lds + (key_a + 4 * which) * ks + c * 32 + grp * 8) : zero8;
             },
             [&](int dt) { return *reinterpret_cast<const bf16x8*>(v_lds + (dt * 16 + col) * vs + grp * 8); }, base, lo, pos, rank, width,
             scale, grp);
@@ -588,16 +604,16 @@ __global__ void __launch_bounds__(256)
       const bf16* ka = cache + (page * PAGE_TOKENS + in_page + key_a) * width + grp * 8;
       const bf16* vt = vt_cache + (page * rank + col) * PAGE_TOKENS + in_page + grp * 8;
       // straight from global memory: half a tile of key loads, then half its latent loads, in flight at once (all of them up to medium sizes)
-      latent_tile<RT, WC, (WC <= 10 ? WC : 9), (RT <= 16 ? RT : 16)>(
+      latent_tile<RT, WC, (WC <= 10 ? WC : 9), (RT <= 16 ? RT : 16), EXACT>(
           st, load_q,
           [&](int which, int c) {
-            return c * 32 + grp * 8 < width ? *reinterpret_cast<const bf16x8*>(ka + which * 4 * (size_t)width + c * 32) : zero8;
+            return (EXACT || c * 32 + grp * 8 < width) ? *reinterpret_cast<const bf16x8*>(ka + which * 4 * (size_t)width + c * 32) : zero8;
           },
           [&](int dt) { return *reinterpret_cast<const bf16x8*>(vt + (size_t)dt * 16 * PAGE_TOKENS); }, base, lo, pos, rank, width, scale,
           grp);
     }
   }
-  latent_finish<RT, WC>(st, out, ldo, ws, t, head, nheads, rank, n_parts, part, grp);
+  latent_finish<RT, WC, EXACT>(st, out, ldo, ws, t, head, nheads, rank, n_parts, part, grp);
 }
 
 // out[t, h, :] = sum_i acc_i exp(m_i - M) / sum_i l_i exp(m_i - M) over the parts i.  The parts' maxima and sums are
@@ -667,14 +683,14 @@ extern "C" int fmsamd_latent_attn_mfma(const void* qa, long ldq, void* out, long
   FMS_REQUIRE(tiles <= 0x7fffffffL && grid.y <= 65535, "latent_attn_mfma: too many tiles for one launch");
   // LDS: every wave's queries; for prompts also a tile of 32 key rows and the same keys' latent, transposed, which the
   // waves of a block share
-#define LAUNCH_LATENT(RT, WC)                                                                                                      \
+#define LAUNCH_LATENT(RT, WC, EXACT)                                                                                               \
   const size_t q_lds = (size_t)4 * WC * 64 * 8 * sizeof(bf16); /* the four waves' queries */                                       \
   const size_t lds = q_lds + (size_t)(32 * (width + 8) + rank * 40) * sizeof(bf16);                                                \
   static bool allowed = false; /* more than 64 KB of LDS a block has to be asked for, once a kernel */                             \
   if (!allowed) {                                                                                                                  \
-    hipError_t e1 = hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<RT, WC, true>,                                        \
+    hipError_t e1 = hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<RT, WC, true, EXACT>,                                 \
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                                   \
-    hipError_t e2 = hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<RT, WC, false>,                                       \
+    hipError_t e2 = hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<RT, WC, false, EXACT>,                                \
                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                                   \
     FMS_REQUIRE(e1 == hipSuccess && e2 == hipSuccess, "latent_attn_mfma: the kernel's LDS could not be sized: %s",                 \
                 hipGetErrorString(e1 != hipSuccess ? e1 : e2));                                                                    \
@@ -682,21 +698,23 @@ extern "C" int fmsamd_latent_attn_mfma(const void* qa, long ldq, void* out, long
   }                                                                                                                                \
   FMS_REQUIRE(lds <= 160 * 1024, "latent_attn_mfma: %zu bytes of LDS", lds);                                                       \
   if (n_splits == 0)                                                                                                               \
-    latent_attn_mfma_kernel<RT, WC, true><<<grid, 256, lds, stream>>>((const bf16*)qa, ldq, (bf16*)out, ldo, (float*)workspace,   \
-                                                                      positions, seq_of_token, block_table, table_stride,         \
-                                                                      (const bf16*)cache, (const bf16*)vt_cache, sink, n_tokens,  \
-                                                                      nheads, rank, width, scale, window, tiles_per_token, n_parts); \
+    latent_attn_mfma_kernel<RT, WC, true, EXACT><<<grid, 256, lds, stream>>>(                                                      \
+        (const bf16*)qa, ldq, (bf16*)out, ldo, (float*)workspace, positions, seq_of_token, block_table, table_stride,              \
+        (const bf16*)cache, (const bf16*)vt_cache, sink, n_tokens, nheads, rank, width, scale, window, tiles_per_token, n_parts);  \
   else                                                                                                                             \
-    latent_attn_mfma_kernel<RT, WC, false><<<grid, 256, q_lds, stream>>>((const bf16*)qa, ldq, (bf16*)out, ldo, (float*)workspace,    \
-                                                                     positions, seq_of_token, block_table, table_stride,          \
-                                                                     (const bf16*)cache, (const bf16*)vt_cache, sink, n_tokens,   \
-                                                                     nheads, rank, width, scale, window, tiles_per_token, n_parts)
-  if (rank <= 128 && width <= 192) {
-    LAUNCH_LATENT(8, 6);
+    latent_attn_mfma_kernel<RT, WC, false, EXACT><<<grid, 256, q_lds, stream>>>(                                                   \
+        (const bf16*)qa, ldq, (bf16*)out, ldo, (float*)workspace, positions, seq_of_token, block_table, table_stride,              \
+        (const bf16*)cache, (const bf16*)vt_cache, sink, n_tokens, nheads, rank, width, scale, window, tiles_per_token, n_parts)
+  // the sizes of the largest configuration exactly (a latent of 512 with a rotated part of 64) run without a question
+  // around any product; everything else in the smallest configuration that holds it
+  if (rank == 512 && width == 576) {
+    LAUNCH_LATENT(32, 18, true);
+  } else if (rank <= 128 && width <= 192) {
+    LAUNCH_LATENT(8, 6, false);
   } else if (rank <= 256 && width <= 320) {
-    LAUNCH_LATENT(16, 10);
+    LAUNCH_LATENT(16, 10, false);
   } else {
-    LAUNCH_LATENT(32, 18);
+    LAUNCH_LATENT(32, 18, false);
   }
 #undef LAUNCH_LATENT
   FMS_LAUNCH_CHECK("latent_attn_mfma");

@@ -631,6 +631,31 @@ def test_command_line_and_trace_replay(lib, folders, tmp_path):
         judge(read(10), want["x"][89:90], dtype)
 
 
+def test_the_inference_program_on_a_zodolorn_folder(lib, folders):
+    """bin/fms_inference with a Zodolorn folder and with a registered variant: the model class comes from config.json or
+    from the registry, the text printed is the plain implementation's greedy continuation."""
+    from fms_amd.tokenizers import CharTokenizer
+
+    name = "A"  # its vocabulary holds the character tokenizer's
+    cfg, weights = plain(folders, name)
+    tok = CharTokenizer()
+    prompt = [ord(c) for c in "latent keys"]
+    new = Z.greedy_generate(cfg, weights, prompt, 12)
+    if tok.eos_token_id in new:
+        new = new[: new.index(tok.eos_token_id)]
+    env = dict(os.environ, PYTHONIOENCODING="utf-8")
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "fms_inference"), "--architecture", "hf_pretrained", "--model_path", folders[name],
+           "--tokenizer", "char_tokenizer", "--default_dtype", "fp32", "--max_new_tokens", "12", "--prompt_ids", ",".join(map(str, prompt))]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=110, env=env)
+    assert proc.returncode == 0, proc.stderr.decode(errors="replace")
+    assert tok.decode(prompt + new) in proc.stdout.decode("utf-8")
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "fms_inference"), "--architecture", "zodolorn", "--variant", "micro", "--tokenizer",
+           "char_tokenizer", "--default_dtype", "bf16", "--max_new_tokens", "5", "--prompt_ids", "1,2,3", "--prompt_ids", "7,8"]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=110, env=env)
+    assert proc.returncode == 0, proc.stderr.decode(errors="replace")
+    assert "loading complete" in proc.stdout.decode("utf-8")
+
+
 def test_a_model_from_the_registry_alone(lib):
     """A registered variant with random weights runs: configuration -> parts -> engine, no folder."""
     from fms_amd.engine import Engine
