@@ -619,10 +619,11 @@ __global__ void __launch_bounds__(256)
 // out[t, h, :] = sum_i acc_i exp(m_i - M) / sum_i l_i exp(m_i - M) over the parts i.  The parts' maxima and sums are
 // loaded side by side (a thread a part) and their weights left in LDS: no chain of dependent loads.
 #define LAT_MAX_PARTS 256
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(256)
     latent_attn_merge_kernel(const float* __restrict__ ws, bf16* __restrict__ out, long ldo, const int* __restrict__ seq_of_token,
                              int nheads, int rank, int n_parts) {
   __shared__ float weight[LAT_MAX_PARTS];
+  __shared__ float inv_total;
   const int h = blockIdx.x, t = blockIdx.y;
   bf16* o = out + (size_t)t * ldo + (size_t)h * rank;
   if (seq_of_token[t] < 0) {
@@ -630,18 +631,21 @@ __global__ void __launch_bounds__(64)
     return;
   }
   const float* w = ws + ((size_t)t * nheads + h) * n_parts * (rank + 4);
-  float top = LAT_EMPTY;
-  for (int i = threadIdx.x; i < n_parts; i += WAVE) top = fmaxf(top, w[(size_t)i * (rank + 4)]);
-  top = wave_max(top);
-  float total = 0.f;
-  for (int i = threadIdx.x; i < n_parts; i += WAVE) {
-    const float e = __expf(w[(size_t)i * (rank + 4)] - top);
-    weight[i] = e;
-    total += w[(size_t)i * (rank + 4) + 1] * e;
+  if (threadIdx.x < WAVE) {  // the first wave weighs the parts
+    float top = LAT_EMPTY;
+    for (int i = threadIdx.x; i < n_parts; i += WAVE) top = fmaxf(top, w[(size_t)i * (rank + 4)]);
+    top = wave_max(top);
+    float total = 0.f;
+    for (int i = threadIdx.x; i < n_parts; i += WAVE) {
+      const float e = __expf(w[(size_t)i * (rank + 4)] - top);
+      weight[i] = e;
+      total += w[(size_t)i * (rank + 4) + 1] * e;
+    }
+    total = wave_sum(total);
+    if (threadIdx.x == 0) inv_total = total > 0.f ? 1.f / total : 0.f;
   }
-  total = wave_sum(total);
   __syncthreads();
-  const float inv = total > 0.f ? 1.f / total : 0.f;
+  const float inv = inv_total;
   for (int d = threadIdx.x; d < rank; d += blockDim.x) {
     float v = 0.f;
 #pragma unroll 8
@@ -719,7 +723,7 @@ extern "C" int fmsamd_latent_attn_mfma(const void* qa, long ldq, void* out, long
 #undef LAUNCH_LATENT
   FMS_LAUNCH_CHECK("latent_attn_mfma");
   if (n_parts > 1) {
-    latent_attn_merge_kernel<<<dim3(nheads, n_tokens), 64, 0, stream>>>((const float*)workspace, (bf16*)out, ldo, seq_of_token, nheads,
+    latent_attn_merge_kernel<<<dim3(nheads, n_tokens), rank > 128 ? 256 : 64, 0, stream>>>((const float*)workspace, (bf16*)out, ldo, seq_of_token, nheads,
                                                                          rank, n_parts);
     FMS_LAUNCH_CHECK("latent_attn_merge");
   }
