@@ -349,11 +349,46 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// The same for rows of at most 256 * KEEP elements: a thread's elements wait in registers and every choice's row is
+// asked for at once, so the kernel pays the memory's latency once a choice instead of once an element and choice.
+template <typename T, int KEEP>
+__global__ void __launch_bounds__(256)
+    combine_small_kernel(const float* __restrict__ y, const float* __restrict__ weights, int top, const T* __restrict__ shared,
+                         const float* __restrict__ shared_gate, long ldg, T* __restrict__ out, int width) {
+  const int t = blockIdx.x;
+  float acc[KEEP], sh[KEEP];
+#pragma unroll
+  for (int n = 0; n < KEEP; ++n) {
+    const int i = threadIdx.x + n * 256;
+    acc[n] = 0.f;
+    sh[n] = (shared && i < width) ? to_f32(shared[(size_t)t * width + i]) : 0.f;
+  }
+  const float sg = shared ? (shared_gate ? 1.f / (1.f + expf(-shared_gate[(size_t)t * ldg])) : 1.f) : 0.f;
+  for (int j = 0; j < top; ++j) {
+    const float wj = weights[(size_t)t * top + j];
+    const float* row = y + ((size_t)t * top + j) * width;
+#pragma unroll
+    for (int n = 0; n < KEEP; ++n) {
+      const int i = threadIdx.x + n * 256;
+      if (i < width) acc[n] = fmaf(wj, row[i], acc[n]);
+    }
+  }
+#pragma unroll
+  for (int n = 0; n < KEEP; ++n) {
+    const int i = threadIdx.x + n * 256;
+    if (i < width) out[(size_t)t * width + i] = from_f32<T>(fmaf(sg, sh[n], acc[n]));
+  }
+}
+
 extern "C" int fmsamd_moe_combine(const float* y, const float* weights, int top, const void* shared, const float* shared_gate,
                                   long ldg, void* out, int dtype, int n_tokens, int width, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   FMS_REQUIRE(n_tokens > 0 && top > 0 && width > 0, "moe_combine: bad sizes T=%d top=%d width=%d", n_tokens, top, width);
-  if (dtype == FMS_F32)
+  if (width <= 256 * 8 && dtype == FMS_F32)
+    combine_small_kernel<float, 8><<<n_tokens, 256, 0, stream>>>(y, weights, top, (const float*)shared, shared_gate, ldg, (float*)out, width);
+  else if (width <= 256 * 8 && dtype == FMS_BF16)
+    combine_small_kernel<bf16, 8><<<n_tokens, 256, 0, stream>>>(y, weights, top, (const bf16*)shared, shared_gate, ldg, (bf16*)out, width);
+  else if (dtype == FMS_F32)
     combine_kernel<float><<<n_tokens, 256, 0, stream>>>(y, weights, top, (const float*)shared, shared_gate, ldg, (float*)out, width);
   else if (dtype == FMS_BF16)
     combine_kernel<bf16><<<n_tokens, 256, 0, stream>>>(y, weights, top, (const bf16*)shared, shared_gate, ldg, (bf16*)out, width);

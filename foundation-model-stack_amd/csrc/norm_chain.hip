@@ -48,11 +48,10 @@ __global__ void __launch_bounds__(256)
 // The same for rows of at most 256 * KEEP elements: branch, stream and both weights are asked for at once and wait in
 // registers, so the kernel pays the memory's latency once instead of four times (a decode step's rows are few, and
 // nothing else hides it).  The loops over what is kept have compile-time trip counts.
-template <typename T, int KEEP>
+template <typename T, typename WT, int KEEP>
 __global__ void __launch_bounds__(256)
-    norm_add_norm_small_kernel(float* __restrict__ resid, const T* __restrict__ branch, const void* __restrict__ wb, float eps_b,
-                               const void* __restrict__ w, int w_dtype, float eps, T* __restrict__ out,
-                               const int* __restrict__ rows, int width) {
+    norm_add_norm_small_kernel(float* __restrict__ resid, const T* __restrict__ branch, const WT* __restrict__ wb, float eps_b,
+                               const WT* __restrict__ w, float eps, T* __restrict__ out, const int* __restrict__ rows, int width) {
   __shared__ float scratch[17];
   const int r = rows ? rows[blockIdx.x] : blockIdx.x;
   float* x = resid + (size_t)r * width;
@@ -66,8 +65,8 @@ __global__ void __launch_bounds__(256)
     if (i < width) {
       bv[n] = to_f32(b[i]);
       xv[n] = x[i];
-      wbv[n] = load_scale(wb, w_dtype, i);
-      wv[n] = load_scale(w, w_dtype, i);
+      if (wb) wbv[n] = to_f32(wb[i]);
+      if (w) wv[n] = to_f32(w[i]);
     }
     sq = fmaf(bv[n], bv[n], sq);
   }
@@ -99,13 +98,17 @@ extern "C" int fmsamd_norm_add_norm(float* resid, const void* branch, int act_dt
   FMS_REQUIRE(n_out > 0 && width > 0 && width <= 16384, "norm_add_norm: bad sizes rows=%d width=%d", n_out, width);
   FMS_REQUIRE(resid != nullptr && branch != nullptr, "norm_add_norm: the stream and the branch are needed");
   const size_t lds = (size_t)width * sizeof(float);
-  if (width <= 256 * 8 && (act_dtype == FMS_F32 || act_dtype == FMS_BF16)) {
-    if (act_dtype == FMS_F32)
-      norm_add_norm_small_kernel<float, 8><<<n_out, 256, 0, stream>>>(resid, (const float*)branch, branch_weight, branch_eps, weight,
-                                                                       weight_dtype, eps, (float*)out, rows, width);
-    else
-      norm_add_norm_small_kernel<bf16, 8><<<n_out, 256, 0, stream>>>(resid, (const bf16*)branch, branch_weight, branch_eps, weight,
-                                                                      weight_dtype, eps, (bf16*)out, rows, width);
+  const bool no_weights = branch_weight == nullptr && weight == nullptr;
+  if (width <= 256 * 8 && (act_dtype == FMS_F32 || act_dtype == FMS_BF16) &&
+      (no_weights || weight_dtype == FMS_F32 || weight_dtype == FMS_BF16)) {
+#define SMALL(T, WT)                                                                                                    \
+  norm_add_norm_small_kernel<T, WT, 8><<<n_out, 256, 0, stream>>>(resid, (const T*)branch, (const WT*)branch_weight, branch_eps, \
+                                                                  (const WT*)weight, eps, (T*)out, rows, width)
+    if (act_dtype == FMS_F32 && (no_weights || weight_dtype == FMS_F32)) SMALL(float, float);
+    else if (act_dtype == FMS_F32) SMALL(float, bf16);
+    else if (no_weights || weight_dtype == FMS_BF16) SMALL(bf16, bf16);
+    else SMALL(bf16, float);
+#undef SMALL
     FMS_LAUNCH_CHECK("norm_add_norm");
     return 0;
   }
