@@ -254,7 +254,7 @@ def _latent_cache(lib, n_pages, width, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("sizes", [(3, 24, 8, 0), (2, 40, 4, 70), (5, 128, 32, 0), (20, 96, 16, 0), (17, 32, 8, 100), (2, 512, 64, 0)])
+@pytest.mark.parametrize("sizes", [(3, 24, 8, 0), (2, 40, 4, 70), (5, 128, 32, 0), (20, 96, 16, 0), (17, 32, 8, 100), (2, 512, 64, 0), (4, 192, 32, 0), (3, 384, 64, 50), (6, 256, 64, 0), (1, 16, 0, 0)])
 def test_attention_over_a_latent_cache(lib, dtype, sizes):
     """Two sequences whose pages lie mixed in the pool; queries of the second at its last positions, the first one
     decoded alone; a sink that matters; one query and one far key scaled so that the far key decides."""
