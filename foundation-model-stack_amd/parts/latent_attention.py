@@ -69,8 +69,9 @@ class LatentAttention(Mixer):
         self._uk_t = self._uv = self._sink = None
         self._mfma = False  # decided when the model's type is known (finalize)
 
-    def fused_parameters(self) -> dict:
-        """The fused down-projection as the tensors it is made of, in the order of its rows."""
+    def unfused_parameters(self) -> dict:
+        """The fused down-projection as the tensors it is made of, in the order of its rows (what the model's
+        state_dict(fused_weights=False) shows in its place)."""
         H = self.nheads
         pieces = [("dq", self.q_rank)] + ([("g", H)] if self.has_gate else []) + ([("dkv", self.kv_rank + self.rot_dim)] if self.owns_kv else [])
         return {"down": tuple(pieces)}
