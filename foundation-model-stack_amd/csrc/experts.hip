@@ -349,19 +349,28 @@ __global__ void __launch_bounds__(256)
   }
 }
 
-// The same for rows of at most 256 * KEEP elements: a thread's elements wait in registers and every choice's row is
-// asked for at once, so the kernel pays the memory's latency once a choice instead of once an element and choice.
+// The same for rows of at most 1024 * KEEP elements (a multiple of 4): a thread's elements wait in registers, four a
+// load, and every choice's row is asked for at once, so the kernel pays the memory's latency once a choice instead of
+// once an element and choice.
 template <typename T, int KEEP>
 __global__ void __launch_bounds__(256)
     combine_small_kernel(const float* __restrict__ y, const float* __restrict__ weights, int top, const T* __restrict__ shared,
                          const float* __restrict__ shared_gate, long ldg, T* __restrict__ out, int width) {
   const int t = blockIdx.x;
-  float acc[KEEP], sh[KEEP];
+  f32x4 acc[KEEP], sh[KEEP];
 #pragma unroll
   for (int n = 0; n < KEEP; ++n) {
-    const int i = threadIdx.x + n * 256;
-    acc[n] = 0.f;
-    sh[n] = (shared && i < width) ? to_f32(shared[(size_t)t * width + i]) : 0.f;
+    const int i = (threadIdx.x + n * 256) * 4;
+    acc[n] = f32x4{0.f, 0.f, 0.f, 0.f};
+    sh[n] = acc[n];
+    if (shared && i < width) {
+      if constexpr (sizeof(T) == 4) {
+        sh[n] = *reinterpret_cast<const f32x4*>(shared + (size_t)t * width + i);
+      } else {
+        const bf16x4 v = *reinterpret_cast<const bf16x4*>(shared + (size_t)t * width + i);
+        sh[n] = f32x4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+      }
+    }
   }
   const float sg = shared ? (shared_gate ? 1.f / (1.f + expf(-shared_gate[(size_t)t * ldg])) : 1.f) : 0.f;
   for (int j = 0; j < top; ++j) {
@@ -369,14 +378,27 @@ __global__ void __launch_bounds__(256)
     const float* row = y + ((size_t)t * top + j) * width;
 #pragma unroll
     for (int n = 0; n < KEEP; ++n) {
-      const int i = threadIdx.x + n * 256;
-      if (i < width) acc[n] = fmaf(wj, row[i], acc[n]);
+      const int i = (threadIdx.x + n * 256) * 4;
+      if (i < width) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(row + i);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[n][e] = fmaf(wj, v[e], acc[n][e]);
+      }
     }
   }
 #pragma unroll
   for (int n = 0; n < KEEP; ++n) {
-    const int i = threadIdx.x + n * 256;
-    if (i < width) out[(size_t)t * width + i] = from_f32<T>(fmaf(sg, sh[n], acc[n]));
+    const int i = (threadIdx.x + n * 256) * 4;
+    if (i < width) {
+      f32x4 r;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) r[e] = fmaf(sg, sh[n][e], acc[n][e]);
+      if constexpr (sizeof(T) == 4) {
+        *reinterpret_cast<f32x4*>(out + (size_t)t * width + i) = r;
+      } else {
+        *reinterpret_cast<bf16x4*>(out + (size_t)t * width + i) = bf16x4{(bf16)r[0], (bf16)r[1], (bf16)r[2], (bf16)r[3]};
+      }
+    }
   }
 }
 
@@ -384,10 +406,10 @@ extern "C" int fmsamd_moe_combine(const float* y, const float* weights, int top,
                                   long ldg, void* out, int dtype, int n_tokens, int width, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   FMS_REQUIRE(n_tokens > 0 && top > 0 && width > 0, "moe_combine: bad sizes T=%d top=%d width=%d", n_tokens, top, width);
-  if (width <= 256 * 8 && dtype == FMS_F32)
-    combine_small_kernel<float, 8><<<n_tokens, 256, 0, stream>>>(y, weights, top, (const float*)shared, shared_gate, ldg, (float*)out, width);
-  else if (width <= 256 * 8 && dtype == FMS_BF16)
-    combine_small_kernel<bf16, 8><<<n_tokens, 256, 0, stream>>>(y, weights, top, (const bf16*)shared, shared_gate, ldg, (bf16*)out, width);
+  if (width <= 1024 * 4 && width % 4 == 0 && dtype == FMS_F32)
+    combine_small_kernel<float, 4><<<n_tokens, 256, 0, stream>>>(y, weights, top, (const float*)shared, shared_gate, ldg, (float*)out, width);
+  else if (width <= 1024 * 4 && width % 4 == 0 && dtype == FMS_BF16)
+    combine_small_kernel<bf16, 4><<<n_tokens, 256, 0, stream>>>(y, weights, top, (const bf16*)shared, shared_gate, ldg, (bf16*)out, width);
   else if (dtype == FMS_F32)
     combine_kernel<float><<<n_tokens, 256, 0, stream>>>(y, weights, top, (const float*)shared, shared_gate, ldg, (float*)out, width);
   else if (dtype == FMS_BF16)

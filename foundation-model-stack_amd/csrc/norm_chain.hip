@@ -45,9 +45,29 @@ __global__ void __launch_bounds__(256)
   for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = from_f32<T>(row[i] * rs * load_scale(w, w_dtype, i));
 }
 
-// The same for rows of at most 256 * KEEP elements: branch, stream and both weights are asked for at once and wait in
-// registers, so the kernel pays the memory's latency once instead of four times (a decode step's rows are few, and
-// nothing else hides it).  The loops over what is kept have compile-time trip counts.
+// Four consecutive elements as floats, from float or bfloat16 storage, in one load; and back.
+template <typename T>
+__device__ __forceinline__ f32x4 load4(const T* p) {
+  if constexpr (sizeof(T) == 4) {
+    return *reinterpret_cast<const f32x4*>(p);
+  } else {
+    const bf16x4 t = *reinterpret_cast<const bf16x4*>(p);
+    return f32x4{(float)t[0], (float)t[1], (float)t[2], (float)t[3]};
+  }
+}
+template <typename T>
+__device__ __forceinline__ void store4(T* p, f32x4 v) {
+  if constexpr (sizeof(T) == 4) {
+    *reinterpret_cast<f32x4*>(p) = v;
+  } else {
+    *reinterpret_cast<bf16x4*>(p) = bf16x4{(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
+  }
+}
+
+// The same for rows of at most 1024 * KEEP elements (a multiple of 4): branch, stream and both weights are asked for
+// at once, four elements a load, and wait in registers, so the kernel pays the memory's latency once instead of four
+// times (a decode step's rows are few, and nothing else hides it).  The loops over what is kept have compile-time
+// trip counts.
 template <typename T, typename WT, int KEEP>
 __global__ void __launch_bounds__(256)
     norm_add_norm_small_kernel(float* __restrict__ resid, const T* __restrict__ branch, const WT* __restrict__ wb, float eps_b,
@@ -56,38 +76,46 @@ __global__ void __launch_bounds__(256)
   const int r = rows ? rows[blockIdx.x] : blockIdx.x;
   float* x = resid + (size_t)r * width;
   const T* b = branch + (size_t)r * width;
-  float bv[KEEP], xv[KEEP], wbv[KEEP], wv[KEEP];
+  const f32x4 ones = {1.f, 1.f, 1.f, 1.f}, zeros = {0.f, 0.f, 0.f, 0.f};
+  f32x4 bv[KEEP], xv[KEEP], wbv[KEEP], wv[KEEP];
   float sq = 0.f;
 #pragma unroll
   for (int n = 0; n < KEEP; ++n) {
-    const int i = threadIdx.x + n * 256;
-    bv[n] = 0.f, xv[n] = 0.f, wbv[n] = 1.f, wv[n] = 1.f;
+    const int i = (threadIdx.x + n * 256) * 4;
+    bv[n] = zeros, xv[n] = zeros, wbv[n] = ones, wv[n] = ones;
     if (i < width) {
-      bv[n] = to_f32(b[i]);
-      xv[n] = x[i];
-      if (wb) wbv[n] = to_f32(wb[i]);
-      if (w) wv[n] = to_f32(w[i]);
+      bv[n] = load4(b + i);
+      xv[n] = load4(x + i);
+      if (wb) wbv[n] = load4(wb + i);
+      if (w) wv[n] = load4(w + i);
     }
-    sq = fmaf(bv[n], bv[n], sq);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) sq = fmaf(bv[n][e], bv[n][e], sq);
   }
   const float rb = rsqrtf(block_sum(sq, scratch) / (float)width + eps_b);
   sq = 0.f;
 #pragma unroll
   for (int n = 0; n < KEEP; ++n) {
-    const int i = threadIdx.x + n * 256;
-    xv[n] = xv[n] + bv[n] * rb * wbv[n];
-    if (i < width) {
-      if (!rows) x[i] = xv[n];
-      sq = fmaf(xv[n], xv[n], sq);
+    const int i = (threadIdx.x + n * 256) * 4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      xv[n][e] = xv[n][e] + bv[n][e] * rb * wbv[n][e];
+      sq = fmaf(xv[n][e], xv[n][e], sq);  // elements past the row are zero
     }
+    if (i < width && !rows) store4(x + i, xv[n]);
   }
   if (out == nullptr) return;
   const float rs = rsqrtf(block_sum(sq, scratch) / (float)width + eps);
   T* o = out + (size_t)blockIdx.x * width;
 #pragma unroll
   for (int n = 0; n < KEEP; ++n) {
-    const int i = threadIdx.x + n * 256;
-    if (i < width) o[i] = from_f32<T>(xv[n] * rs * wv[n]);
+    const int i = (threadIdx.x + n * 256) * 4;
+    if (i < width) {
+      f32x4 y;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) y[e] = xv[n][e] * rs * wv[n][e];
+      store4(o + i, y);
+    }
   }
 }
 
@@ -99,10 +127,10 @@ extern "C" int fmsamd_norm_add_norm(float* resid, const void* branch, int act_dt
   FMS_REQUIRE(resid != nullptr && branch != nullptr, "norm_add_norm: the stream and the branch are needed");
   const size_t lds = (size_t)width * sizeof(float);
   const bool no_weights = branch_weight == nullptr && weight == nullptr;
-  if (width <= 256 * 8 && (act_dtype == FMS_F32 || act_dtype == FMS_BF16) &&
+  if (width <= 1024 * 4 && width % 4 == 0 && (act_dtype == FMS_F32 || act_dtype == FMS_BF16) &&
       (no_weights || weight_dtype == FMS_F32 || weight_dtype == FMS_BF16)) {
 #define SMALL(T, WT)                                                                                                    \
-  norm_add_norm_small_kernel<T, WT, 8><<<n_out, 256, 0, stream>>>(resid, (const T*)branch, (const WT*)branch_weight, branch_eps, \
+  norm_add_norm_small_kernel<T, WT, 4><<<n_out, 256, 0, stream>>>(resid, (const T*)branch, (const WT*)branch_weight, branch_eps, \
                                                                   (const WT*)weight, eps, (T*)out, rows, width)
     if (act_dtype == FMS_F32 && (no_weights || weight_dtype == FMS_F32)) SMALL(float, float);
     else if (act_dtype == FMS_F32) SMALL(float, bf16);

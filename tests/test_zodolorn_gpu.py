@@ -183,7 +183,7 @@ def judge(got, want, dtype):
 
 # ---- mechanisms alone ------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("width", [40, 192, 1000, 3000])
+@pytest.mark.parametrize("width", [40, 192, 1001, 3000, 4100])
 def test_norm_behind_a_branch_sum_and_next_norm(lib, dtype, width):
     from fms_amd.kernels import ops
 
@@ -329,7 +329,7 @@ def test_router(lib, sizes):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("sizes", [(6, 2, 48, 128, 50), (5, 1, 36, 100, 7), (8, 8, 128, 256, 40), (3, 2, 20, 64, 1), (4, 2, 64, 128, 300), (3, 3, 200, 72, 150), (2, 2, 16, 2304, 3)])
+@pytest.mark.parametrize("sizes", [(6, 2, 48, 128, 50), (5, 1, 36, 100, 7), (8, 8, 128, 256, 40), (3, 2, 20, 64, 1), (4, 2, 64, 128, 300), (3, 3, 200, 72, 150), (2, 2, 16, 4352, 3), (3, 1, 24, 70, 9)])
 def test_experts_and_their_sum(lib, dtype, sizes):
     from fms_amd.kernels import ops
 
