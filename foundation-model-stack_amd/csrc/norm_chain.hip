@@ -188,9 +188,31 @@ __global__ void activate_kernel(const T* __restrict__ x, T* __restrict__ out, lo
     out[i] = from_f32<T>(fms_activate(to_f32(x[i]), act));
 }
 
+// four elements a thread and step, for element counts that are multiples of 4
+template <typename T>
+__global__ void activate4_kernel(const T* __restrict__ x, T* __restrict__ out, long n4, int act) {
+  const long stride = (long)gridDim.x * blockDim.x;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
+    f32x4 v = load4(x + 4 * i);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = fms_activate(v[e], act);
+    store4(out + 4 * i, v);
+  }
+}
+
 extern "C" int fmsamd_activate(const void* x, void* out, int dtype, long n, int act, hipStream_t stream) {
   if (n == 0) return 0;
   FMS_REQUIRE(n > 0 && act >= 0 && act <= FMS_ACT_LAST, "activate: bad arguments n=%ld act=%d", n, act);
+  if (n % 4 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)out % 16) == 0 && (dtype == FMS_F32 || dtype == FMS_BF16)) {
+    const long n4 = n / 4;
+    const int blocks4 = (int)((n4 + 255) / 256 < 8192 ? (n4 + 255) / 256 : 8192);
+    if (dtype == FMS_F32)
+      activate4_kernel<float><<<blocks4, 256, 0, stream>>>((const float*)x, (float*)out, n4, act);
+    else
+      activate4_kernel<bf16><<<blocks4, 256, 0, stream>>>((const bf16*)x, (bf16*)out, n4, act);
+    FMS_LAUNCH_CHECK("activate");
+    return 0;
+  }
   const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
   if (dtype == FMS_F32)
     activate_kernel<float><<<blocks, 256, 0, stream>>>((const float*)x, (float*)out, n, act);
@@ -208,7 +230,21 @@ __device__ __forceinline__ float clamped_gate(float g, float u, float limit, flo
   return g / (1.f + expf(-alpha * g)) * (u + shift);
 }
 
-// gu [T, 2 * hidden] (gate first), out [T, hidden]
+// gu [T, 2 * hidden] (gate first), out [T, hidden]; hidden a multiple of 4: four elements a thread and step
+template <typename T>
+__global__ void clamped_gated_act4_kernel(const T* __restrict__ gu, T* __restrict__ out, int hidden, float limit, float alpha,
+                                          float shift) {
+  const T* g = gu + (size_t)blockIdx.x * 2 * hidden;
+  T* o = out + (size_t)blockIdx.x * hidden;
+  for (int i = threadIdx.x * 4; i < hidden; i += blockDim.x * 4) {
+    const f32x4 gv = load4(g + i), uv = load4(g + hidden + i);
+    f32x4 r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) r[e] = clamped_gate(gv[e], uv[e], limit, alpha, shift);
+    store4(o + i, r);
+  }
+}
+
 template <typename T>
 __global__ void clamped_gated_act_kernel(const T* __restrict__ gu, T* __restrict__ out, int hidden, float limit,
                                          float alpha, float shift) {
@@ -223,6 +259,14 @@ extern "C" int fmsamd_clamped_gated_act(const void* gu, void* out, int dtype, in
   if (n_tokens == 0) return 0;
   FMS_REQUIRE(n_tokens > 0 && hidden > 0 && limit > 0.f, "clamped_gated_act: bad arguments T=%d hidden=%d limit=%g", n_tokens,
               hidden, (double)limit);
+  if (hidden % 4 == 0 && ((uintptr_t)gu % 16) == 0 && ((uintptr_t)out % 16) == 0 && (dtype == FMS_F32 || dtype == FMS_BF16)) {
+    if (dtype == FMS_F32)
+      clamped_gated_act4_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)gu, (float*)out, hidden, limit, alpha, shift);
+    else
+      clamped_gated_act4_kernel<bf16><<<n_tokens, 256, 0, stream>>>((const bf16*)gu, (bf16*)out, hidden, limit, alpha, shift);
+    FMS_LAUNCH_CHECK("clamped_gated_act");
+    return 0;
+  }
   if (dtype == FMS_F32)
     clamped_gated_act_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)gu, (float*)out, hidden, limit, alpha, shift);
   else if (dtype == FMS_BF16)

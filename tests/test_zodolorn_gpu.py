@@ -216,15 +216,16 @@ def test_embedding_with_a_scale(lib):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_activations_beside_the_gated_ones(lib, dtype):
+@pytest.mark.parametrize("hidden", [33, 36])  # single elements, and four a load
+def test_activations_beside_the_gated_ones(lib, dtype, hidden):
     from fms_amd.kernels import ops
 
-    x = (torch.randn(9, 70) * 3).to(dtype)
+    x = (torch.randn(9, 2 * hidden + 1 if hidden % 4 else 2 * hidden) * 3).to(dtype)
     tol = dict(atol=1e-6, rtol=1e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=1e-2)
     xf = x.float()
     torch.testing.assert_close(ops.activation(x.to(DEV), "gelu").float().cpu(), 0.5 * xf * (1 + torch.erf(xf / math.sqrt(2))), **tol)
-    gu = (torch.randn(9, 2 * 33) * 3).to(dtype)
-    g, u = gu.float()[:, :33].clamp(max=1.5), gu.float()[:, 33:].clamp(-1.5, 1.5)
+    gu = (torch.randn(9, 2 * hidden) * 3).to(dtype)
+    g, u = gu.float()[:, :hidden].clamp(max=1.5), gu.float()[:, hidden:].clamp(-1.5, 1.5)
     want = g * torch.sigmoid(1.702 * g) * (u + 1.0)
     torch.testing.assert_close(ops.clamped_gated_act(gu.to(DEV), 1.5, 1.702, 1.0).float().cpu(), want, **tol)
     assert float((gu.float().abs() > 1.5).float().mean()) > 0.3  # the limits were reached
