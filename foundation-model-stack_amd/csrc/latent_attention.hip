@@ -179,6 +179,32 @@ __global__ void __launch_bounds__(TILE_THREADS) headwise_mfma_kernel(HeadwiseArg
   }
 }
 
+// The same on tiles of 64 tokens (a wave 32 x 64), for steps of many tokens: a head's weights are read once for 64
+// tokens instead of once for 16.
+__global__ void __launch_bounds__(TILE_THREADS) headwise_mfma_wide_kernel(HeadwiseArgs a) {
+  const int t0 = blockIdx.x * TILE_WIDE_ROWS, h = blockIdx.y, n0 = blockIdx.z * TILE_MFMA_COLS;
+  const bf16* x = (const bf16*)a.x + (size_t)h * a.xs;
+  const bf16* w = (const bf16*)a.w + (size_t)h * a.N * a.K;
+  f32x4 acc[2][4];
+  tile_product_mfma_wide([&](int m) { return t0 + m < a.T ? x + (size_t)(t0 + m) * a.ldx : (const bf16*)nullptr; },
+                         [&](int n) { return n0 + n < a.N ? w + (size_t)(n0 + n) * a.K : (const bf16*)nullptr; }, a.K, acc);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int t = t0 + (wave >> 1) * 32 + mt * 16 + (lane >> 4) * 4 + i;
+      if (t >= a.T) continue;
+      const float g = a.gate ? 1.f / (1.f + expf(-a.gate[(size_t)t * a.ldg + h])) : 1.f;
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) {
+        const int n = n0 + (wave & 1) * 64 + nt * 16 + (lane & 15);
+        if (n < a.N) ((bf16*)a.y)[(size_t)t * a.ldy + (size_t)h * a.ys + n] = (bf16)(acc[mt][nt][i] * g);
+      }
+    }
+  }
+}
+
 extern "C" int fmsamd_headwise_linear(const void* x, long ldx, long x_head_stride, const void* w, void* y, long ldy,
                                       long y_head_stride, const float* gate, long ldg, int dtype, int n_tokens, int nheads,
                                       int N, int K, hipStream_t stream) {
@@ -193,7 +219,9 @@ extern "C" int fmsamd_headwise_linear(const void* x, long ldx, long x_head_strid
     headwise_fma_kernel<float><<<dim3(row_tiles, nheads, ceil_div(N, TILE_FMA_COLS)), TILE_THREADS, 0, stream>>>(a);
   } else if (dtype == FMS_BF16) {
     const bool aligned = K % 8 == 0 && ldx % 8 == 0 && x_head_stride % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0;
-    if (aligned)
+    if (aligned && n_tokens >= 2 * TILE_WIDE_ROWS)
+      headwise_mfma_wide_kernel<<<dim3(ceil_div(n_tokens, TILE_WIDE_ROWS), nheads, ceil_div(N, TILE_MFMA_COLS)), TILE_THREADS, 0, stream>>>(a);
+    else if (aligned)
       headwise_mfma_kernel<<<dim3(row_tiles, nheads, ceil_div(N, TILE_MFMA_COLS)), TILE_THREADS, 0, stream>>>(a);
     else
       headwise_fma_kernel<bf16><<<dim3(row_tiles, nheads, ceil_div(N, TILE_FMA_COLS)), TILE_THREADS, 0, stream>>>(a);

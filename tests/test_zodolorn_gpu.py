@@ -232,7 +232,7 @@ def test_activations_beside_the_gated_ones(lib, dtype, hidden):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("shape", [(5, 3, 12, 28), (37, 4, 16, 40), (20, 8, 64, 128), (3, 2, 128, 48)])
+@pytest.mark.parametrize("shape", [(5, 3, 12, 28), (37, 4, 16, 40), (20, 8, 64, 128), (3, 2, 128, 48), (150, 3, 64, 136), (129, 2, 40, 24)])
 def test_a_product_per_head(lib, dtype, shape):
     from fms_amd.kernels import ops
 
