@@ -24,6 +24,9 @@ class Architecture:
     to_hf_dict: Callable[[ModelConfig], dict] = None
     hf_tensor_layout: Callable[[ModelConfig], list] = None  # names/shapes/inits of a Hugging Face checkpoint
     detect_source: Callable[[list], str] = None  # a checkpoint's tensor names -> the name of its source (adapter)
+    # (configuration, checkpoint tensor name -> shape) -> configuration: for sizes that a model folder gives only as
+    # shapes of its tensors
+    sizes_from_tensors: Callable[[ModelConfig, dict], ModelConfig] = None
 
 
 _architectures: Dict[str, Architecture] = {}

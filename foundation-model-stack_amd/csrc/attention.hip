@@ -29,7 +29,7 @@ __global__ void __launch_bounds__(GEN_THREADS)
     attn_generic_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ out, long out_stride,
                         const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                         const int* __restrict__ block_table, int table_stride, const T* __restrict__ k_cache,
-                        const T* __restrict__ v_cache, int nheads, int kvheads, int head_dim, float scale, int window,
+                        const T* __restrict__ v_cache, int nheads, int kvheads, int head_dim, int vdim, float scale, int window,
                         const float* __restrict__ slopes, float soft_cap) {
   __shared__ float qs[256];
   __shared__ float ps[GEN_THREADS];
@@ -37,9 +37,9 @@ __global__ void __launch_bounds__(GEN_THREADS)
   const int h = blockIdx.x;
   const int t = blockIdx.y;
   const int seq = seq_of_token[t];
-  T* o = out + (size_t)t * out_stride + (size_t)h * head_dim;
+  T* o = out + (size_t)t * out_stride + (size_t)h * vdim;  // values (and so the output) may have a size of their own
   if (seq < 0) {
-    for (int d = threadIdx.x; d < head_dim; d += blockDim.x) o[d] = from_f32<T>(0.f);
+    for (int d = threadIdx.x; d < vdim; d += blockDim.x) o[d] = from_f32<T>(0.f);
     return;
   }
   const int pos = positions[t];
@@ -47,6 +47,7 @@ __global__ void __launch_bounds__(GEN_THREADS)
   const int kh = h / (nheads / kvheads);
   const int* bt = block_table + (size_t)seq * table_stride;
   const size_t page_elems = (size_t)kvheads * PAGE_TOKENS * head_dim;
+  const size_t vpage_elems = (size_t)kvheads * PAGE_TOKENS * vdim;
 
   const T* qrow = q + (size_t)t * q_stride + (size_t)h * head_dim;
   for (int d = threadIdx.x; d < head_dim; d += blockDim.x) qs[d] = to_f32(qrow[d]);
@@ -74,21 +75,21 @@ __global__ void __launch_bounds__(GEN_THREADS)
     const float psum = block_sum(p, scratch);  // has the barriers that publish ps
     l_run = l_run * alpha + psum;
     m_run = m_new;
-    if ((int)threadIdx.x < head_dim) {
+    if ((int)threadIdx.x < vdim) {
       const int d = threadIdx.x;
       float a = acc * alpha;
       const int n = pos - base + 1 < GEN_THREADS ? pos - base + 1 : GEN_THREADS;
       for (int i = 0; i < n; ++i) {
         const int jj = base + i;
-        const T* vrow = v_cache + readable_page(bt[jj / PAGE_TOKENS]) * page_elems +
-                        ((size_t)kh * head_dim + d) * PAGE_TOKENS + jj % PAGE_TOKENS;
+        const T* vrow = v_cache + readable_page(bt[jj / PAGE_TOKENS]) * vpage_elems +
+                        ((size_t)kh * vdim + d) * PAGE_TOKENS + jj % PAGE_TOKENS;
         a = fmaf(ps[i], to_f32(*vrow), a);
       }
       acc = a;
     }
     __syncthreads();  // ps is overwritten by the next chunk
   }
-  if ((int)threadIdx.x < head_dim) o[threadIdx.x] = from_f32<T>(l_run > 0.f ? acc / l_run : 0.f);
+  if ((int)threadIdx.x < vdim) o[threadIdx.x] = from_f32<T>(l_run > 0.f ? acc / l_run : 0.f);
 }
 
 #define LOG2E 1.4426950408889634f
@@ -1251,9 +1252,11 @@ extern "C" int fmsamd_attn_generic(const void* q, long q_stride, void* out, long
                                    const int* positions, const int* seq_of_token, const int* block_table,
                                    int table_stride, const void* k_cache, const void* v_cache, int n_tokens,
                                    int nheads, int kvheads, int head_dim, float scale, int window,
-                                   const float* slopes, float soft_cap, hipStream_t stream) {
+                                   const float* slopes, float soft_cap, int value_dim, hipStream_t stream) {
   if (n_tokens == 0) return 0;
-  if (check_common("attn_generic", n_tokens, nheads, kvheads, head_dim, q_stride, out_stride)) return -1;
+  const int vdim = value_dim > 0 ? value_dim : head_dim;
+  if (check_common("attn_generic", n_tokens, nheads, kvheads, head_dim, q_stride, vdim == head_dim ? out_stride : q_stride)) return -1;
+  FMS_REQUIRE(vdim <= 256 && out_stride >= (long)nheads * vdim, "attn_generic: value size %d is above 256 or the output rows are too short", vdim);
   FMS_REQUIRE(n_tokens <= 65535, "attn_generic: %d tokens exceed one launch (65535)", n_tokens);
   FMS_REQUIRE(soft_cap >= 0.f, "attn_generic: soft cap %g is negative", (double)soft_cap);
   dim3 grid(nheads, n_tokens);
@@ -1261,7 +1264,7 @@ extern "C" int fmsamd_attn_generic(const void* q, long q_stride, void* out, long
 #define FMS_GEN(T, TERMS)                                                                                              \
   attn_generic_kernel<T, TERMS><<<grid, GEN_THREADS, 0, stream>>>(                                                     \
       (const T*)q, q_stride, (T*)out, out_stride, positions, seq_of_token, block_table, table_stride, (const T*)k_cache, \
-      (const T*)v_cache, nheads, kvheads, head_dim, scale, window, slopes, soft_cap)
+      (const T*)v_cache, nheads, kvheads, head_dim, vdim, scale, window, slopes, soft_cap)
   if (dtype == FMS_F32) {
     if (terms)
       FMS_GEN(float, true);

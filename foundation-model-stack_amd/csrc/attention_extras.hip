@@ -1,0 +1,88 @@
+// Steps around attention that some mixers have and others do not:
+//   qk_projection_norm: an RMS norm over the whole query projection and one over the whole key projection (all heads
+//                       at once, before they are cut into heads and rotated), from the float32 sums of the projection;
+//                       the values are copied.  One rounding to the activation type.
+//   gate_mul:           out = x * act(gate) * scale (gate: float32 logits, or none), into rows of any stride.
+//   scale_f32:          x *= s in place.
+#include "common.h"
+#include "fmsamd.h"
+
+template <typename T, typename W>
+__global__ void __launch_bounds__(256)
+    qk_projection_norm_kernel(const float* __restrict__ proj, long ld, int nq, int nk, int nv, const W* __restrict__ wq,
+                              const W* __restrict__ wk, float eps, T* __restrict__ out, long ldo,
+                              const int* __restrict__ seq_of_token) {
+  __shared__ float scratch[17];
+  const int t = blockIdx.x;
+  if (seq_of_token != nullptr && seq_of_token[t] < 0) return;
+  const float* row = proj + (size_t)t * ld;
+  T* o = out + (size_t)t * ldo;
+  float sq = 0.f, sk = 0.f;
+  for (int i = threadIdx.x; i < nq; i += blockDim.x) sq = fmaf(row[i], row[i], sq);
+  for (int i = threadIdx.x; i < nk; i += blockDim.x) sk = fmaf(row[nq + i], row[nq + i], sk);
+  sq = block_sum(sq, scratch);
+  sk = block_sum(sk, scratch);
+  const float iq = 1.f / sqrtf(sq / (float)nq + eps), ik = 1.f / sqrtf(sk / (float)nk + eps);
+  for (int i = threadIdx.x; i < nq; i += blockDim.x) o[i] = from_f32<T>(row[i] * iq * (wq ? to_f32(wq[i]) : 1.f));
+  for (int i = threadIdx.x; i < nk; i += blockDim.x) o[nq + i] = from_f32<T>(row[nq + i] * ik * (wk ? to_f32(wk[i]) : 1.f));
+  for (int i = threadIdx.x; i < nv; i += blockDim.x) o[nq + nk + i] = from_f32<T>(row[nq + nk + i]);
+}
+
+extern "C" int fmsamd_qk_projection_norm(const float* proj, long ld, int nq, int nk, int nv, const void* wq, const void* wk,
+                                         int weight_dtype, float eps, void* out, int out_dtype, long ldo, const int* seq_of_token,
+                                         int n_tokens, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  FMS_REQUIRE(n_tokens > 0 && nq > 0 && nk > 0 && nv >= 0 && ld >= (long)nq + nk + nv && ldo >= (long)nq + nk + nv,
+              "qk_projection_norm: bad sizes q=%d k=%d v=%d", nq, nk, nv);
+#define FMS_QKN(T, W)                                                                                                        \
+  qk_projection_norm_kernel<T, W><<<n_tokens, 256, 0, stream>>>(proj, ld, nq, nk, nv, (const W*)wq, (const W*)wk, eps, (T*)out, \
+                                                                ldo, seq_of_token)
+  if (out_dtype == FMS_F32 && weight_dtype == FMS_F32) FMS_QKN(float, float);
+  else if (out_dtype == FMS_BF16 && weight_dtype == FMS_F32) FMS_QKN(bf16, float);
+  else if (out_dtype == FMS_BF16 && weight_dtype == FMS_BF16) FMS_QKN(bf16, bf16);
+  else if (out_dtype == FMS_F32 && weight_dtype == FMS_BF16) FMS_QKN(float, bf16);
+  else FMS_REQUIRE(false, "qk_projection_norm: unknown dtypes %d, %d", out_dtype, weight_dtype);
+#undef FMS_QKN
+  FMS_LAUNCH_CHECK("qk_projection_norm");
+  return 0;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+    gate_mul_kernel(const T* __restrict__ x, long ldx, const float* __restrict__ gate, long ldg, int act, float scale,
+                    T* __restrict__ out, long ldo, int cols) {
+  const int t = blockIdx.x;
+  for (int i = threadIdx.x; i < cols; i += blockDim.x) {
+    float v = to_f32(x[(size_t)t * ldx + i]) * scale;
+    if (gate != nullptr) v *= fms_activate(gate[(size_t)t * ldg + i], act);
+    out[(size_t)t * ldo + i] = from_f32<T>(v);
+  }
+}
+
+extern "C" int fmsamd_gate_mul(const void* x, long ldx, const float* gate, long ldg, int act, float scale, void* out, long ldo,
+                               int dtype, int n_tokens, int cols, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  FMS_REQUIRE(n_tokens > 0 && cols > 0 && ldx >= cols && ldo >= cols && (gate == nullptr || ldg >= cols), "gate_mul: bad sizes");
+  FMS_REQUIRE(act >= 0 && act <= FMS_ACT_LAST, "gate_mul: unknown activation %d", act);
+  if (dtype == FMS_F32)
+    gate_mul_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)x, ldx, gate, ldg, act, scale, (float*)out, ldo, cols);
+  else if (dtype == FMS_BF16)
+    gate_mul_kernel<bf16><<<n_tokens, 256, 0, stream>>>((const bf16*)x, ldx, gate, ldg, act, scale, (bf16*)out, ldo, cols);
+  else
+    FMS_REQUIRE(false, "gate_mul: unknown dtype %d", dtype);
+  FMS_LAUNCH_CHECK("gate_mul");
+  return 0;
+}
+
+__global__ void __launch_bounds__(256) scale_f32_kernel(float* __restrict__ x, size_t n, float s) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) x[i] *= s;
+}
+
+extern "C" int fmsamd_scale_f32(float* x, long n, float s, hipStream_t stream) {
+  if (n == 0) return 0;
+  FMS_REQUIRE(n > 0, "scale_f32: negative count");
+  const int blocks = ceil_div(n, 256) > 4096 ? 4096 : ceil_div(n, 256);
+  scale_f32_kernel<<<blocks, 256, 0, stream>>>(x, (size_t)n, s);
+  FMS_LAUNCH_CHECK("scale_f32");
+  return 0;
+}

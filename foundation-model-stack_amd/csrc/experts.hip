@@ -1,7 +1,8 @@
 // A feed-forward of many small experts of which every token uses a few.
 //
-//   route:    float32 router logits [T, E] -> the `top` largest per token (ties: the lower index) and the softmax over
-//             those `top` logits alone.
+//   route:    float32 router logits [T, E] -> the `top` largest per token (ties: the lower index) and their weights:
+//             the softmax over those `top` logits alone, or every chosen logit's sigmoid (as it is, or divided by the
+//             sum of the chosen ones).
 //   group:    the T * top (token, choice) pairs sorted by expert, cut into tiles of 16 rows that belong to one expert
 //             each.  It runs on the device, in one block, so a step never waits for the host (and can be captured).
 //   gate_up:  for every tile, hidden = clamp-gated activation of (x Wg_e^T, x Wu_e^T)
@@ -20,7 +21,7 @@
 
 // One wave per token.
 __global__ void __launch_bounds__(256)
-    route_kernel(const float* __restrict__ logits, long ld, int n_tokens, int n_experts, int top, int* __restrict__ ids,
+    route_kernel(const float* __restrict__ logits, long ld, int n_tokens, int n_experts, int top, int score, int* __restrict__ ids,
                  float* __restrict__ weights) {
   extern __shared__ float lds[];  // 4 waves x (n_experts + top)
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -53,21 +54,29 @@ __global__ void __launch_bounds__(256)
     __threadfence_block();
   }
   if (lane == 0) {
-    const float m = chosen[0];  // the largest comes first
-    float sum = 0.f;
-    for (int j = 0; j < top; ++j) sum += expf(chosen[j] - m);
-    for (int j = 0; j < top; ++j) weights[(size_t)t * top + j] = expf(chosen[j] - m) / sum;
+    if (score == FMS_ROUTE_SOFTMAX) {
+      const float m = chosen[0];  // the largest comes first
+      float sum = 0.f;
+      for (int j = 0; j < top; ++j) sum += expf(chosen[j] - m);
+      for (int j = 0; j < top; ++j) weights[(size_t)t * top + j] = expf(chosen[j] - m) / sum;
+    } else {  // sigmoid scores (the order of the logits is the order of their sigmoids)
+      float sum = 0.f;
+      for (int j = 0; j < top; ++j) sum += 1.f / (1.f + expf(-chosen[j]));
+      const float norm = score == FMS_ROUTE_SIGMOID_NORMED ? 1.f / sum : 1.f;
+      for (int j = 0; j < top; ++j) weights[(size_t)t * top + j] = norm / (1.f + expf(-chosen[j]));
+    }
   }
 }
 
-extern "C" int fmsamd_moe_route(const float* logits, long ld, int n_tokens, int n_experts, int top, int* ids, float* weights,
-                                hipStream_t stream) {
+extern "C" int fmsamd_moe_route(const float* logits, long ld, int n_tokens, int n_experts, int top, int score, int* ids,
+                                float* weights, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   FMS_REQUIRE(n_tokens > 0 && n_experts > 0 && n_experts <= ROUTE_MAX_EXPERTS && top > 0 && top <= n_experts && top <= ROUTE_MAX_TOP,
               "moe_route: %d experts (at most %d), top %d (at most %d and the experts)", n_experts, ROUTE_MAX_EXPERTS, top, ROUTE_MAX_TOP);
   FMS_REQUIRE(ld >= n_experts, "moe_route: rows of %ld for %d experts", ld, n_experts);
+  FMS_REQUIRE(score >= FMS_ROUTE_SOFTMAX && score <= FMS_ROUTE_SIGMOID_NORMED, "moe_route: unknown score %d", score);
   const size_t lds = 4 * (size_t)(n_experts + top) * sizeof(float);
-  route_kernel<<<ceil_div(n_tokens, 4), 256, lds, stream>>>(logits, ld, n_tokens, n_experts, top, ids, weights);
+  route_kernel<<<ceil_div(n_tokens, 4), 256, lds, stream>>>(logits, ld, n_tokens, n_experts, top, score, ids, weights);
   FMS_LAUNCH_CHECK("moe_route");
   return 0;
 }
@@ -145,7 +154,12 @@ struct ExpertArgs {
   const int* tiles;
   int top, N, K;
   float limit, alpha, shift;
+  const float* in_scale;  // gate_up: a factor per pair on the expert's input (applied to both float32 sums), or null
 };
+
+__device__ __forceinline__ float pair_scale(const ExpertArgs& a, int sorted_row) {
+  return a.in_scale ? a.in_scale[a.order[sorted_row]] : 1.f;
+}
 
 __device__ __forceinline__ float clamp_gated(float g, float u, float limit, float alpha, float shift) {
   g = fminf(g, limit);
@@ -170,7 +184,10 @@ __global__ void __launch_bounds__(TILE_THREADS) expert_gate_up_fma_kernel(Expert
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int m = (threadIdx.x / 64) * 4 + i;
-    if (m < rows) ((T*)a.y)[(size_t)(start + m) * a.N + n] = from_f32<T>(clamp_gated(g[i], u[i], a.limit, a.alpha, a.shift));
+    if (m < rows) {
+      const float sc = pair_scale(a, start + m);
+      ((T*)a.y)[(size_t)(start + m) * a.N + n] = from_f32<T>(clamp_gated(g[i] * sc, u[i] * sc, a.limit, a.alpha, a.shift));
+    }
   }
 }
 
@@ -209,10 +226,11 @@ __global__ void __launch_bounds__(TILE_THREADS) expert_gate_up_mfma_kernel(Exper
   for (int i = 0; i < 4; ++i) {
     const int m = (lane >> 4) * 4 + i;
     if (m >= rows) continue;
+    const float sc = pair_scale(a, start + m);
 #pragma unroll
     for (int tl = 0; tl < TILE_MFMA_WAVE_TILES; ++tl) {
       const int n = n0 + wave * (16 * TILE_MFMA_WAVE_TILES) + tl * 16 + (lane & 15);
-      if (n < a.N) ((bf16*)a.y)[(size_t)(start + m) * a.N + n] = (bf16)clamp_gated(g[tl][i], u[tl][i], a.limit, a.alpha, a.shift);
+      if (n < a.N) ((bf16*)a.y)[(size_t)(start + m) * a.N + n] = (bf16)clamp_gated(g[tl][i] * sc, u[tl][i] * sc, a.limit, a.alpha, a.shift);
     }
   }
 }
@@ -259,10 +277,11 @@ __global__ void __launch_bounds__(TILE_THREADS) expert_gate_up_wide_kernel(Exper
     for (int i = 0; i < 4; ++i) {
       const int m = (wave >> 1) * 32 + mt * 16 + (lane >> 4) * 4 + i;
       if (m >= rows) continue;
+      const float sc = pair_scale(a, start + m);
 #pragma unroll
       for (int nt = 0; nt < 4; ++nt) {
         const int n = n0 + (wave & 1) * 64 + nt * 16 + (lane & 15);
-        if (n < a.N) ((bf16*)a.y)[(size_t)(start + m) * a.N + n] = (bf16)clamp_gated(g[mt][nt][i], u[mt][nt][i], a.limit, a.alpha, a.shift);
+        if (n < a.N) ((bf16*)a.y)[(size_t)(start + m) * a.N + n] = (bf16)clamp_gated(g[mt][nt][i] * sc, u[mt][nt][i] * sc, a.limit, a.alpha, a.shift);
       }
     }
   }
@@ -298,13 +317,13 @@ __global__ void __launch_bounds__(TILE_THREADS) expert_down_wide_kernel(ExpertAr
 // tile_rows: what fmsamd_moe_tile_rows said when the tiles were made
 extern "C" int fmsamd_moe_experts(int stage, const void* x, long ldx, const void* w1, const void* w2, void* y, int dtype,
                                   const int* order, const int* tiles, int max_tiles, int tile_rows, int top, int N, int K,
-                                  float limit, float alpha, float shift, hipStream_t stream) {
+                                  float limit, float alpha, float shift, const float* in_scale, hipStream_t stream) {
   if (max_tiles == 0) return 0;
   FMS_REQUIRE(stage == 0 || stage == 1, "moe_experts: stage %d", stage);
   FMS_REQUIRE(tile_rows == TILE_ROWS || tile_rows == TILE_WIDE_ROWS, "moe_experts: tiles of %d rows", tile_rows);
   FMS_REQUIRE(max_tiles > 0 && top > 0 && N > 0 && K > 0 && ldx >= K, "moe_experts: bad sizes tiles=%d top=%d N=%d K=%d ldx=%ld", max_tiles,
               top, N, K, ldx);
-  ExpertArgs a{x, ldx, w1, w2, y, order, tiles, top, N, K, limit, alpha, shift};
+  ExpertArgs a{x, ldx, w1, w2, y, order, tiles, top, N, K, limit, alpha, shift, stage == 0 ? in_scale : nullptr};
   const bool mfma = dtype == FMS_BF16 && K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w1 % 16) == 0 &&
                     (w2 == nullptr || ((uintptr_t)w2 % 16) == 0);
   const dim3 grid(max_tiles, ceil_div(N, mfma ? TILE_MFMA_COLS : TILE_FMA_COLS));
@@ -343,7 +362,7 @@ __global__ void __launch_bounds__(256)
   const float sg = shared ? (shared_gate ? 1.f / (1.f + expf(-shared_gate[(size_t)t * ldg])) : 1.f) : 0.f;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     float v = 0.f;
-    for (int j = 0; j < top; ++j) v = fmaf(weights[(size_t)t * top + j], y[((size_t)t * top + j) * width + i], v);
+    for (int j = 0; j < top; ++j) v = fmaf(weights ? weights[(size_t)t * top + j] : 1.f, y[((size_t)t * top + j) * width + i], v);
     if (shared) v = fmaf(sg, to_f32(shared[(size_t)t * width + i]), v);
     out[(size_t)t * width + i] = from_f32<T>(v);
   }
@@ -374,7 +393,7 @@ __global__ void __launch_bounds__(256)
   }
   const float sg = shared ? (shared_gate ? 1.f / (1.f + expf(-shared_gate[(size_t)t * ldg])) : 1.f) : 0.f;
   for (int j = 0; j < top; ++j) {
-    const float wj = weights[(size_t)t * top + j];
+    const float wj = weights ? weights[(size_t)t * top + j] : 1.f;  // no weights: the plain sum
     const float* row = y + ((size_t)t * top + j) * width;
 #pragma unroll
     for (int n = 0; n < KEEP; ++n) {

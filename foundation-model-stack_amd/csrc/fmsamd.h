@@ -6,7 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define FMSAMD_ABI_VERSION 3
+#define FMSAMD_ABI_VERSION 4
 
 // element types
 #define FMS_F32 0
@@ -54,19 +54,21 @@ int fmsamd_bias_add(void* x, int dtype, const void* bias, int bias_dtype, int ro
 int fmsamd_rope_table(const float* freqs, float* cos_t, float* sin_t, int max_pos, int half, hipStream_t stream);
 
 // Rotate the queries of qkv in place; rotate the keys and write keys and values into the paged cache
-// (k_cache/v_cache null: queries only).  cos_t null: no rotation.
+// (k_cache/v_cache null: queries only).  cos_t null: no rotation.  value_dim (0: head_dim): the size of a value if it
+// is not the size of a key; the rows are then [H*D | K*D | K*value_dim] and the value pages [kv head][value_dim][token].
 int fmsamd_rope_kv_write(void* qkv, int dtype, long row_stride, const int* positions, const int* seq_of_token,
                          const int* block_table, int table_stride, const float* cos_t, const float* sin_t,
                          int rot_dim, int max_pos, void* k_cache, void* v_cache, int n_tokens, int nheads, int kvheads,
-                         int head_dim, hipStream_t stream);
+                         int head_dim, int value_dim, hipStream_t stream);
 
 // causal attention over the cache; any element type, any even head size up to 256.  Further terms of the scores:
 // slopes (float32 [nheads] or null): score += slopes[head] * (key position - query position); soft_cap (0: none):
-// score = soft_cap * tanh(score / soft_cap), before the slope term.
+// score = soft_cap * tanh(score / soft_cap), before the slope term.  value_dim (0: head_dim): values and output heads
+// of another size than the keys.
 int fmsamd_attn_generic(const void* q, long q_stride, void* out, long out_stride, int dtype, const int* positions,
                         const int* seq_of_token, const int* block_table, int table_stride, const void* k_cache,
                         const void* v_cache, int n_tokens, int nheads, int kvheads, int head_dim, float scale,
-                        int window, const float* slopes, float soft_cap, hipStream_t stream);
+                        int window, const float* slopes, float soft_cap, int value_dim, hipStream_t stream);
 
 // bfloat16 prefill: the step is cut into query blocks of at most fmsamd_attn_prefill_qblock(...) consecutive
 // tokens of one sequence; the same number goes into the call as qblock_tokens
@@ -216,7 +218,12 @@ int fmsamd_latent_attn_mfma(const void* qa, long ldq, void* out, long ldo, void*
                             int rot, float scale, int window, int n_splits, hipStream_t stream);
 
 // ---- experts (experts.hip) -----------------------------------------------------------------------------------------
-int fmsamd_moe_route(const float* logits, long ld, int n_tokens, int n_experts, int top, int* ids, float* weights,
+// ids: the `top` largest logits of every token; weights: FMS_ROUTE_SOFTMAX the softmax over the chosen logits,
+// FMS_ROUTE_SIGMOID each chosen logit's sigmoid, FMS_ROUTE_SIGMOID_NORMED those divided by their sum.
+#define FMS_ROUTE_SOFTMAX 0
+#define FMS_ROUTE_SIGMOID 1
+#define FMS_ROUTE_SIGMOID_NORMED 2
+int fmsamd_moe_route(const float* logits, long ld, int n_tokens, int n_experts, int top, int score, int* ids, float* weights,
                      hipStream_t stream);
 // Rows of a tile of (token, choice) pairs of one expert: 64 where experts have many rows and the matrix-core kernel can
 // run (wide_ok), else 16; the most tiles there can be; the pairs sorted by expert and cut into tiles:
@@ -225,12 +232,45 @@ int fmsamd_moe_tile_rows(int n_pairs, int n_experts, int wide_ok);
 int fmsamd_moe_max_tiles(int n_pairs, int n_experts, int tile_rows);
 int fmsamd_moe_group(const int* ids, int n_pairs, int n_experts, int* order, int* tiles, int max_tiles, int tile_rows,
                      hipStream_t stream);
-// stage 0: y[sorted pair] = act(x Wg^T, x Wu^T) (w1, w2 = gate, up [E, N, K]); stage 1: y[pair] = x W^T, float32
+// stage 0: y[sorted pair] = act(s x Wg^T, s x Wu^T) (w1, w2 = gate, up [E, N, K]; s = in_scale[pair], or 1 if null: a
+// weight on the expert's input, applied to the float32 sums); stage 1: y[pair] = x W^T, float32
 int fmsamd_moe_experts(int stage, const void* x, long ldx, const void* w1, const void* w2, void* y, int dtype,
                        const int* order, const int* tiles, int max_tiles, int tile_rows, int top, int N, int K, float limit,
-                       float alpha, float shift, hipStream_t stream);
+                       float alpha, float shift, const float* in_scale, hipStream_t stream);
+// weights null: the plain sum of a token's rows
 int fmsamd_moe_combine(const float* y, const float* weights, int top, const void* shared, const float* shared_gate, long ldg,
                        void* out, int dtype, int n_tokens, int width, hipStream_t stream);
+
+// ---- steps around attention (attention_extras.hip) ------------------------------------------------------------------
+// float32 rows [q (nq) | k (nk) | v (nv)]: out = [q / rms(q) * wq | k / rms(k) * wk | v], each norm over its whole run of
+// columns; rows whose seq_of_token is negative are skipped (seq_of_token null: none are)
+int fmsamd_qk_projection_norm(const float* proj, long ld, int nq, int nk, int nv, const void* wq, const void* wk,
+                              int weight_dtype, float eps, void* out, int out_dtype, long ldo, const int* seq_of_token,
+                              int n_tokens, hipStream_t stream);
+// out = x * act(gate) * scale (gate: float32 logits or null)
+int fmsamd_gate_mul(const void* x, long ldx, const float* gate, long ldg, int act, float scale, void* out, long ldo,
+                    int dtype, int n_tokens, int cols, hipStream_t stream);
+int fmsamd_scale_f32(float* x, long n, float s, hipStream_t stream);
+
+// ---- the gated delta rule (delta_rule.hip) ------------------------------------------------------------------------------
+// proj: float32 rows whose first C = 2*kv_heads*dim + heads*vdim columns are the q, k and v channels before the
+// convolution and whose columns col_b .. col_b + heads are the logits of beta; a: rows with the decay's input at col_a
+// (heads columns, or heads*dim if per_channel); conv_w [C, taps]; conv_state [slots][taps-1][C] is read, then updated.
+// Writes qkv [T, C] (convolved, silu, q and k unit vectors per head, q times q_scale), beta [T, heads] and
+// decay [T, heads (*dim)] = exp(-exp(a_log) softplus(a + dt_bias)).
+int fmsamd_delta_prepare(const float* proj, long ld, int col_b, const float* a, long lda, int col_a, const void* conv_w,
+                         int conv_dtype, int taps, const float* a_log, const float* dt_bias, float* conv_state,
+                         const int* seq_of_token, const int* slot_ids, float* qkv, float* beta, float* decay, int n_tokens,
+                         int heads, int kv_heads, int dim, int vdim, int per_channel, float q_scale, hipStream_t stream);
+// The recurrence over every sequence's tokens of the step (seq_starts [n_seqs + 1]); state [slots][heads][vdim][dim]
+// is read and written; out [T, heads*vdim].
+int fmsamd_delta_rule(const float* qkv, const float* beta, const float* decay, float* state, float* out,
+                      const int* seq_starts, const int* seq_of_token, const int* slot_ids, int n_seqs, int heads,
+                      int kv_heads, int dim, int vdim, int per_channel, hipStream_t stream);
+// out[t, h, :] = o[t, h, :] / rms * weight * act(gate[t, h, :]) * out_scale
+int fmsamd_gated_head_norm(const float* o, const float* gate, long ldg, const void* weight, int weight_dtype, float eps,
+                           int act, float out_scale, void* out, int out_dtype, long ldo, const int* seq_of_token,
+                           int n_tokens, int heads, int vdim, hipStream_t stream);
 
 #ifdef __cplusplus
 }

@@ -38,7 +38,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, long row_stride, const
                                      const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
                                      int table_stride, const float* __restrict__ cos_t,
                                      const float* __restrict__ sin_t, int rot_dim, int max_pos, T* __restrict__ k_cache,
-                                     T* __restrict__ v_cache, int nheads, int kvheads, int head_dim) {
+                                     T* __restrict__ v_cache, int nheads, int kvheads, int head_dim, int vdim) {
   const int t = blockIdx.x;
   const int seq = seq_of_token[t];
   if (seq < 0) return;  // padding row of a fixed-size batch
@@ -56,6 +56,38 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, long row_stride, const
   }
   const size_t page_elems = (size_t)kvheads * PAGE_TOKENS * head_dim;
 
+  if (vdim != head_dim) {
+    // values of a size of their own: the row is [H*D | K*D | K*vdim]; q and k in pairs, then the values one by one
+    for (int idx = threadIdx.x; idx < (nheads + kvheads) * half; idx += blockDim.x) {
+      const int hh = idx / half;
+      const int i = idx % half;
+      T* p = row + (size_t)hh * head_dim + 2 * i;
+      float a = to_f32(p[0]), b = to_f32(p[1]);
+      if (cos_t && i < rot_half) {
+        const float c = cos_t[(size_t)tpos * rot_half + i];
+        const float s = sin_t[(size_t)tpos * rot_half + i];
+        const float ra = c * a - s * b;
+        const float rb = s * a + c * b;
+        a = ra;
+        b = rb;
+      }
+      if (hh < nheads) {
+        p[0] = from_f32<T>(a);
+        p[1] = from_f32<T>(b);
+      } else if (k_cache) {
+        T* dst = k_cache + page * page_elems + ((size_t)(hh - nheads) * PAGE_TOKENS + in_page) * head_dim + 2 * i;
+        dst[0] = from_f32<T>(a);
+        dst[1] = from_f32<T>(b);
+      }
+    }
+    if (v_cache) {
+      const T* vrow = row + (size_t)(nheads + kvheads) * head_dim;
+      const size_t vpage_elems = (size_t)kvheads * PAGE_TOKENS * vdim;
+      for (int idx = threadIdx.x; idx < kvheads * vdim; idx += blockDim.x)
+        v_cache[page * vpage_elems + (size_t)idx * PAGE_TOKENS + in_page] = vrow[idx];
+    }
+    return;
+  }
   const int total = (nheads + 2 * kvheads) * half;
   for (int idx = threadIdx.x; idx < total; idx += blockDim.x) {
     const int hh = idx / half;
@@ -235,14 +267,15 @@ __global__ void __launch_bounds__(256)
 extern "C" int fmsamd_rope_kv_write(void* qkv, int dtype, long row_stride, const int* positions,
                                     const int* seq_of_token, const int* block_table, int table_stride,
                                     const float* cos_t, const float* sin_t, int rot_dim, int max_pos, void* k_cache,
-                                    void* v_cache, int n_tokens, int nheads, int kvheads, int head_dim,
+                                    void* v_cache, int n_tokens, int nheads, int kvheads, int head_dim, int value_dim,
                                     hipStream_t stream) {
   if (n_tokens == 0) return 0;
+  const int vdim = value_dim > 0 ? value_dim : head_dim;
   FMS_REQUIRE(n_tokens > 0 && nheads > 0 && kvheads > 0 && head_dim > 0, "rope_kv_write: bad sizes");
   FMS_REQUIRE(head_dim % 2 == 0, "rope_kv_write: head size %d is odd", head_dim);
   FMS_REQUIRE(rot_dim % 2 == 0 && rot_dim >= 0 && rot_dim <= head_dim, "rope_kv_write: rotary size %d does not fit head size %d",
               rot_dim, head_dim);
-  FMS_REQUIRE(row_stride >= (long)(nheads + 2 * kvheads) * head_dim, "rope_kv_write: row stride too small");
+  FMS_REQUIRE(row_stride >= (long)(nheads + kvheads) * head_dim + (long)kvheads * vdim, "rope_kv_write: row stride too small");
   FMS_REQUIRE((k_cache == nullptr) == (v_cache == nullptr), "rope_kv_write: key and value cache must come together");
   FMS_REQUIRE(cos_t == nullptr || max_pos > 0, "rope_kv_write: empty table");
   const int threads = 256;
@@ -250,7 +283,7 @@ extern "C" int fmsamd_rope_kv_write(void* qkv, int dtype, long row_stride, const
   const size_t elem = dtype == FMS_F32 ? 4 : 2;
   FMS_REQUIRE(dtype == FMS_F32 || dtype == FMS_BF16, "rope_kv_write: unknown dtype %d", dtype);
   // four elements a thread need rows that start at multiples of four elements
-  const bool by_fours = head_dim % 4 == 0 && row_stride % 4 == 0 && (uintptr_t)qkv % (4 * elem) == 0 &&
+  const bool by_fours = vdim == head_dim && head_dim % 4 == 0 && row_stride % 4 == 0 && (uintptr_t)qkv % (4 * elem) == 0 &&
                         (uintptr_t)k_cache % (4 * elem) == 0 && (uintptr_t)v_cache % (4 * elem) == 0;
   if (by_fours) {
     const int rt = dtype == FMS_F32 ? 32 : 64;
@@ -276,11 +309,11 @@ extern "C" int fmsamd_rope_kv_write(void* qkv, int dtype, long row_stride, const
   } else if (dtype == FMS_F32)
     rope_kv_write_kernel<float><<<n_tokens, threads, 0, stream>>>(
         (float*)qkv, row_stride, positions, seq_of_token, block_table, table_stride, c, sin_t, rot_dim, max_pos,
-        (float*)k_cache, (float*)v_cache, nheads, kvheads, head_dim);
+        (float*)k_cache, (float*)v_cache, nheads, kvheads, head_dim, vdim);
   else
     rope_kv_write_kernel<bf16><<<n_tokens, threads, 0, stream>>>(
         (bf16*)qkv, row_stride, positions, seq_of_token, block_table, table_stride, c, sin_t, rot_dim, max_pos,
-        (bf16*)k_cache, (bf16*)v_cache, nheads, kvheads, head_dim);
+        (bf16*)k_cache, (bf16*)v_cache, nheads, kvheads, head_dim, vdim);
   FMS_LAUNCH_CHECK("rope_kv_write");
   return 0;
 }

@@ -17,7 +17,7 @@ import torch  # noqa: F401  (loads libamdhip64 before our library asks for it)
 
 from . import build as _build
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _lib: Optional[ctypes.CDLL] = None
 _lock = threading.Lock()
@@ -32,8 +32,8 @@ _SIGNATURES = {
     "fmsamd_advance_positions": [P, P, I, P],
     "fmsamd_bias_add": [P, I, P, I, I, I, P],
     "fmsamd_rope_table": [P, P, P, I, I, P],
-    "fmsamd_rope_kv_write": [P, I, L, P, P, P, I, P, P, I, I, P, P, I, I, I, I, P],
-    "fmsamd_attn_generic": [P, L, P, L, I, P, P, P, I, P, P, I, I, I, I, F, I, P, F, P],
+    "fmsamd_rope_kv_write": [P, I, L, P, P, P, I, P, P, I, I, P, P, I, I, I, I, I, P],
+    "fmsamd_attn_generic": [P, L, P, L, I, P, P, P, I, P, P, I, I, I, I, F, I, P, F, I, P],
     "fmsamd_attn_prefill_bf16": [P, L, P, L, P, P, P, P, I, I, P, I, P, P, I, I, I, I, F, I, P],
     "fmsamd_attn_decode_bf16": [P, L, P, L, P, L, P, P, P, I, P, P, I, I, I, I, F, I, I, I, I, I, P, P],
     "fmsamd_qkv_rope_skinny_bf16": [P, L, P, P, I, P, L, I, I, P, P, P, I, P, P, I, I, P, P, I, I, I, P, P, L, P],
@@ -56,9 +56,15 @@ _SIGNATURES = {
     "fmsamd_latent_q_rotate": [P, L, I, I, I, I, P, L, I, P, P, P, I, I, P],
     "fmsamd_headwise_linear": [P, L, L, P, P, L, L, P, L, I, I, I, I, I, P],
     "fmsamd_latent_attn_generic": [P, L, P, L, I, P, P, P, I, P, P, I, I, I, I, F, I, P],
-    "fmsamd_moe_route": [P, L, I, I, I, P, P, P],
+    "fmsamd_moe_route": [P, L, I, I, I, I, P, P, P],
     "fmsamd_moe_group": [P, I, I, P, P, I, I, P],
-    "fmsamd_moe_experts": [I, P, L, P, P, P, I, P, P, I, I, I, I, I, F, F, F, P],
+    "fmsamd_moe_experts": [I, P, L, P, P, P, I, P, P, I, I, I, I, I, F, F, F, P, P],
+    "fmsamd_qk_projection_norm": [P, L, I, I, I, P, P, I, F, P, I, L, P, I, P],
+    "fmsamd_gate_mul": [P, L, P, L, I, F, P, L, I, I, I, P],
+    "fmsamd_scale_f32": [P, L, F, P],
+    "fmsamd_delta_prepare": [P, L, I, P, L, I, P, I, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, P],
+    "fmsamd_delta_rule": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
+    "fmsamd_gated_head_norm": [P, P, L, P, I, F, I, F, P, I, L, P, I, I, I, P],
     "fmsamd_moe_combine": [P, P, I, P, P, L, P, I, I, I, P],
     "fmsamd_probe_read": [P, L, I, I, P, P],
     "fmsamd_probe_mfma": [I, I, I, P, P, P],

@@ -166,13 +166,14 @@ def rope_table(freqs: torch.Tensor, max_pos: int):
     return cos, sin
 
 
-def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, kvheads: int, head_dim: int, dtype: torch.dtype) -> int:
+def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, kvheads: int, head_dim: int, dtype: torch.dtype,
+                 value_dim: int = 0) -> int:
     shape = (kvheads, PAGE_TOKENS, head_dim)
     if k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != shape or not k_cache.is_contiguous():
         raise ValueError(f"key cache must be contiguous [pages, {kvheads}, {PAGE_TOKENS}, {head_dim}], got {tuple(k_cache.shape)}")
-    vshape = (kvheads, head_dim, PAGE_TOKENS)
+    vshape = (kvheads, value_dim or head_dim, PAGE_TOKENS)
     if v_cache.dim() != 4 or tuple(v_cache.shape[1:]) != vshape or not v_cache.is_contiguous():
-        raise ValueError(f"value cache must be contiguous [pages, {kvheads}, {head_dim}, {PAGE_TOKENS}], got {tuple(v_cache.shape)}")
+        raise ValueError(f"value cache must be contiguous [pages, {kvheads}, {value_dim or head_dim}, {PAGE_TOKENS}], got {tuple(v_cache.shape)}")
     if k_cache.dtype != dtype or v_cache.dtype != dtype or k_cache.shape[0] != v_cache.shape[0]:
         raise TypeError("key and value cache must have the dtype of the queries and equal page counts")
     return k_cache.shape[0]
@@ -287,8 +288,10 @@ def rope_kv_write(
     nheads: int,
     kvheads: int,
     head_dim: int,
+    value_dim: int = 0,
 ) -> None:
     """Rotate q (in place, inside qkv) and k; write k and v of every token into its cache page.
+    value_dim (0: head_dim): values of a size of their own; the rows are then [H*D | K*D | K*value_dim].
 
     The caller guarantees (and the engine checks on the host) that every position is below the
     table length and that block_table holds a valid page for every (sequence, position // 64).
@@ -296,8 +299,9 @@ def rope_kv_write(
     _need_cuda(qkv, positions, seq_of_token, block_table, cos, sin, k_cache, v_cache)
     _rows2d("qkv", qkv)
     T = qkv.shape[0]
-    if qkv.shape[1] != (nheads + 2 * kvheads) * head_dim:
-        raise ValueError(f"qkv has {qkv.shape[1]} columns, expected {(nheads + 2 * kvheads) * head_dim}")
+    value_dim = 0 if value_dim == head_dim else int(value_dim)
+    if qkv.shape[1] != (nheads + kvheads) * head_dim + kvheads * (value_dim or head_dim):
+        raise ValueError(f"qkv has {qkv.shape[1]} columns, expected {(nheads + kvheads) * head_dim + kvheads * (value_dim or head_dim)}")
     _check_batch_index(positions, seq_of_token, block_table, T)
     max_pos = 0
     if cos is not None:
@@ -307,11 +311,11 @@ def rope_kv_write(
             raise ValueError("cos/sin tables must be contiguous")
         max_pos = cos.shape[0]
     if k_cache is not None:
-        _check_cache(k_cache, v_cache, kvheads, head_dim, qkv.dtype)
+        _check_cache(k_cache, v_cache, kvheads, head_dim, qkv.dtype, value_dim)
     check(load().fmsamd_rope_kv_write(qkv.data_ptr(), _code(qkv.dtype), qkv.stride(0), positions.data_ptr(),
                                       seq_of_token.data_ptr(), block_table.data_ptr(), block_table.stride(0),
                                       _ptr(cos), _ptr(sin), rot_dim if cos is not None else 0, max_pos, _ptr(k_cache),
-                                      _ptr(v_cache), T, nheads, kvheads, head_dim, _stream()))
+                                      _ptr(v_cache), T, nheads, kvheads, head_dim, value_dim, _stream()))
 
 
 def attention(
@@ -339,8 +343,10 @@ def attention(
     row_order: Optional[torch.Tensor] = None,
     score_slopes: Optional[torch.Tensor] = None,
     soft_cap: float = 0.0,
+    value_dim: int = 0,
 ) -> torch.Tensor:
-    """Causal attention of every token over the cache of its sequence -> [T, nheads*head_dim].
+    """Causal attention of every token over the cache of its sequence -> [T, nheads*head_dim] (with value_dim, values
+    and output heads of that size, through the generic kernel).
 
     Further terms of the scores (a position encoding that acts on the scores, a capped attention): score_slopes,
     float32 [nheads], adds slope[head] * (key position - query position); soft_cap c > 0 turns a score s into
@@ -355,8 +361,9 @@ def attention(
     _rows2d("q", q)
     T = q.shape[0]
     _check_batch_index(positions, seq_of_token, block_table, T)
-    _check_cache(k_cache, v_cache, kvheads, head_dim, q.dtype)
-    out = torch.empty(T, nheads * head_dim, dtype=q.dtype, device=q.device)
+    value_dim = 0 if value_dim == head_dim else int(value_dim)
+    _check_cache(k_cache, v_cache, kvheads, head_dim, q.dtype, value_dim)
+    out = torch.empty(T, nheads * (value_dim or head_dim), dtype=q.dtype, device=q.device)
     lib = load()
     common_tail = (T, nheads, kvheads, head_dim, float(scale), int(window), _stream())
     if score_slopes is not None:
@@ -365,13 +372,13 @@ def attention(
             raise ValueError(f"score_slopes must be a contiguous float32 [{nheads}] tensor")
     if not (soft_cap >= 0.0 and math.isfinite(soft_cap)):
         raise ValueError(f"soft_cap {soft_cap} must be zero (none) or positive")
-    if q.dtype == torch.float32 or force_generic or head_dim % 16 or score_slopes is not None or soft_cap > 0.0:
+    if q.dtype == torch.float32 or force_generic or head_dim % 16 or score_slopes is not None or soft_cap > 0.0 or value_dim:
         for t0 in range(0, T, 65535):
             n = min(65535, T - t0)
             check(lib.fmsamd_attn_generic(q[t0:].data_ptr(), q.stride(0), out[t0:].data_ptr(), out.stride(0), _code(q.dtype),
                                           positions[t0:].data_ptr(), seq_of_token[t0:].data_ptr(), block_table.data_ptr(),
                                           block_table.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), n, *common_tail[1:-1],
-                                          _ptr(score_slopes), float(soft_cap), common_tail[-1]))
+                                          _ptr(score_slopes), float(soft_cap), value_dim, common_tail[-1]))
         return out
     if decode:
         if max_context <= 0:
@@ -812,9 +819,13 @@ def latent_attention(qa: torch.Tensor, positions, seq_of_token, block_table, cac
 # --------------------------------------------------------------------------
 # experts
 # --------------------------------------------------------------------------
-def moe_route(logits: torch.Tensor, n_experts: int, top: int):
+ROUTE_SCORES = {"softmax": 0, "sigmoid": 1, "sigmoid_normed": 2}
+
+
+def moe_route(logits: torch.Tensor, n_experts: int, top: int, score: str = "softmax"):
     """float32 logits [T, >= n_experts] -> (int32 ids [T, top], float32 weights [T, top]): the `top` largest logits of
-    every token among the first n_experts columns, and the softmax over those alone."""
+    every token among the first n_experts columns, and their weights: the softmax over those alone ("softmax"), each
+    one's sigmoid ("sigmoid"), or the sigmoids divided by their sum ("sigmoid_normed")."""
     _need_cuda(logits)
     _rows2d("logits", logits)
     if logits.dtype != torch.float32 or logits.shape[1] < n_experts:
@@ -822,15 +833,19 @@ def moe_route(logits: torch.Tensor, n_experts: int, top: int):
     T = logits.shape[0]
     ids = torch.empty(T, top, dtype=torch.int32, device=logits.device)
     weights = torch.empty(T, top, dtype=torch.float32, device=logits.device)
-    check(load().fmsamd_moe_route(logits.data_ptr(), logits.stride(0), T, n_experts, top, ids.data_ptr(), weights.data_ptr(), _stream()))
+    check(load().fmsamd_moe_route(logits.data_ptr(), logits.stride(0), T, n_experts, top, ROUTE_SCORES[score], ids.data_ptr(),
+                                  weights.data_ptr(), _stream()))
     return ids, weights
 
 
 def moe_experts(x: torch.Tensor, ids: torch.Tensor, gate_w: torch.Tensor, up_w: torch.Tensor, down_w: torch.Tensor,
-                limit: float, alpha: float, shift: float) -> torch.Tensor:
+                limit: float, alpha: float, shift: float, in_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Every (token, choice) pair through its expert: float32 [T * top, width], row t * top + j the output of expert
-    ids[t, j] for token t.  gate_w, up_w [E, ff, width], down_w [E, width, ff]."""
-    _need_cuda(x, ids, gate_w, up_w, down_w)
+    ids[t, j] for token t.  gate_w, up_w [E, ff, width], down_w [E, width, ff].  in_scale (float32 [T, top]): a factor
+    on the expert's input for every pair, applied to the float32 sums of the gate and up products."""
+    _need_cuda(x, ids, gate_w, up_w, down_w, in_scale)
+    if in_scale is not None and (in_scale.dtype != torch.float32 or tuple(in_scale.shape) != tuple(ids.shape) or not in_scale.is_contiguous()):
+        raise ValueError("in_scale is a contiguous float32 tensor of the shape of ids")
     _rows2d("x", x)
     _need_i32("ids", ids)
     T, top = ids.shape
@@ -853,19 +868,28 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, gate_w: torch.Tensor, up_w: 
     y = torch.empty(n_pairs, width, dtype=torch.float32, device=x.device)
     code = _code(x.dtype)
     check(lib.fmsamd_moe_experts(0, x.data_ptr(), x.stride(0), gate_w.data_ptr(), up_w.data_ptr(), hidden.data_ptr(), code,
-                                 order.data_ptr(), tiles.data_ptr(), max_tiles, tile_rows, top, ff, width, float(limit), float(alpha), float(shift), _stream()))
+                                 order.data_ptr(), tiles.data_ptr(), max_tiles, tile_rows, top, ff, width, float(limit), float(alpha), float(shift),
+                                 _ptr(in_scale), _stream()))
     check(lib.fmsamd_moe_experts(1, hidden.data_ptr(), hidden.stride(0), down_w.data_ptr(), None, y.data_ptr(), code,
-                                 order.data_ptr(), tiles.data_ptr(), max_tiles, tile_rows, top, width, ff, float(limit), float(alpha), float(shift), _stream()))
+                                 order.data_ptr(), tiles.data_ptr(), max_tiles, tile_rows, top, width, ff, float(limit), float(alpha), float(shift),
+                                 None, _stream()))
     return y
 
 
-def moe_combine(y: torch.Tensor, weights: torch.Tensor, shared: Optional[torch.Tensor], shared_gate: Optional[torch.Tensor],
-                out_dtype: torch.dtype) -> torch.Tensor:
+def moe_combine(y: torch.Tensor, weights: Optional[torch.Tensor], shared: Optional[torch.Tensor], shared_gate: Optional[torch.Tensor],
+                out_dtype: torch.dtype, top: int = 0) -> torch.Tensor:
     """out[t] = sum_j weights[t, j] * y[t * top + j] (+ sigmoid(shared_gate[t]) * shared[t]) in out_dtype.
+    weights None (then `top` says how many rows a token has): the plain sum.
     shared_gate: a float32 column view [T] (any row stride) of logits, or None for an ungated shared output."""
     _need_cuda(y, weights, shared, shared_gate)
-    T, top = weights.shape
-    if y.dtype != torch.float32 or y.dim() != 2 or y.shape[0] != T * top or not y.is_contiguous() or not weights.is_contiguous() or weights.dtype != torch.float32:
+    if weights is not None:
+        T, top = weights.shape
+    elif top <= 0 or y.dim() != 2 or y.shape[0] % top:
+        raise ValueError("moe_combine without weights needs the number of rows a token has")
+    else:
+        T = y.shape[0] // top
+    if y.dtype != torch.float32 or y.dim() != 2 or y.shape[0] != T * top or not y.is_contiguous() or (
+            weights is not None and (not weights.is_contiguous() or weights.dtype != torch.float32)):
         raise ValueError("moe_combine: y is contiguous float32 [T * top, width], weights float32 [T, top]")
     width = y.shape[1]
     if shared is not None and (tuple(shared.shape) != (T, width) or shared.dtype != out_dtype or not shared.is_contiguous()):
@@ -876,8 +900,165 @@ def moe_combine(y: torch.Tensor, weights: torch.Tensor, shared: Optional[torch.T
             raise ValueError("the shared gate is a float32 [T] view and needs a shared output")
         ldg = shared_gate.stride(0)
     out = torch.empty(T, width, dtype=out_dtype, device=y.device)
-    check(load().fmsamd_moe_combine(y.data_ptr(), weights.data_ptr(), top, _ptr(shared), _ptr(shared_gate), ldg, out.data_ptr(),
+    check(load().fmsamd_moe_combine(y.data_ptr(), _ptr(weights), top, _ptr(shared), _ptr(shared_gate), ldg, out.data_ptr(),
                                     _code(out_dtype), T, width, _stream()))
+    return out
+
+
+# --------------------------------------------------------------------------
+# steps around attention
+# --------------------------------------------------------------------------
+def qk_projection_norm(proj: torch.Tensor, nq: int, nk: int, nv: int, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
+                       eps: float, out_dtype: torch.dtype, seq_of_token: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """float32 rows [q (nq) | k (nk) | v (nv) | ...] -> [T, nq + nk + nv] in out_dtype: q and k each RMS-normed over
+    their whole run of columns (all heads at once) times a weight, v as it is."""
+    _need_cuda(proj, q_weight, k_weight, seq_of_token)
+    _rows2d("proj", proj)
+    if proj.dtype != torch.float32 or proj.shape[1] < nq + nk + nv:
+        raise ValueError("qk_projection_norm takes float32 rows that hold queries, keys and values")
+    wdtype = None
+    for n, w in ((nq, q_weight), (nk, k_weight)):
+        if w is not None:
+            if tuple(w.shape) != (n,) or not w.is_contiguous() or (wdtype is not None and w.dtype != wdtype):
+                raise ValueError("the norm weights are contiguous vectors of the projections' sizes and of one type")
+            wdtype = w.dtype
+    if seq_of_token is not None:
+        _need_i32("seq_of_token", seq_of_token)
+    out = torch.empty(proj.shape[0], nq + nk + nv, dtype=out_dtype, device=proj.device)
+    check(load().fmsamd_qk_projection_norm(proj.data_ptr(), proj.stride(0), nq, nk, nv, _ptr(q_weight), _ptr(k_weight),
+                                           _code(wdtype) if wdtype is not None else 0, float(eps), out.data_ptr(), _code(out_dtype),
+                                           out.stride(0), _ptr(seq_of_token), proj.shape[0], _stream()))
+    return out
+
+
+def gate_mul(x: torch.Tensor, gate: Optional[torch.Tensor], activation: str = "sigmoid", scale: float = 1.0,
+             out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x * act(gate) * scale, elementwise over rows [T, cols]; gate: float32 logits (a view with contiguous rows) or None;
+    out: rows of any stride to write into (default: a new tensor)."""
+    _need_cuda(x, gate, out)
+    _rows2d("x", x)
+    T, cols = x.shape
+    if gate is not None:
+        _rows2d("gate", gate)
+        if gate.dtype != torch.float32 or tuple(gate.shape) != (T, cols):
+            raise ValueError(f"the gate is float32 [{T}, {cols}]")
+    if out is None:
+        out = torch.empty(T, cols, dtype=x.dtype, device=x.device)
+    _rows2d("out", out)
+    if out.dtype != x.dtype or tuple(out.shape) != (T, cols):
+        raise ValueError(f"out is [{T}, {cols}] of the type of x")
+    check(load().fmsamd_gate_mul(x.data_ptr(), x.stride(0), _ptr(gate), gate.stride(0) if gate is not None else 0, ACTIVATIONS[activation],
+                                 float(scale), out.data_ptr(), out.stride(0), _code(x.dtype), T, cols, _stream()))
+    return out
+
+
+def scale_(x: torch.Tensor, s: float) -> torch.Tensor:
+    """x *= s in place (contiguous float32)."""
+    _need_cuda(x)
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise ValueError("scale_ takes a contiguous float32 tensor")
+    check(load().fmsamd_scale_f32(x.data_ptr(), x.numel(), float(s), _stream()))
+    return x
+
+
+# --------------------------------------------------------------------------
+# the gated delta rule
+# --------------------------------------------------------------------------
+DELTA_MAX_TAPS = 8
+DELTA_MAX_DIM = 256
+
+
+def delta_prepare(proj: torch.Tensor, col_b: int, a: torch.Tensor, col_a: int, conv_w: torch.Tensor, a_log: torch.Tensor,
+                  dt_bias: torch.Tensor, conv_state: torch.Tensor, seq_of_token: torch.Tensor, slot_ids: torch.Tensor, heads: int,
+                  kv_heads: int, dim: int, vdim: int, per_channel: bool, q_scale: float):
+    """What the recurrence of a step reads, from the float32 projections of its tokens: (qkv [T, C], beta [T, heads],
+    decay [T, heads] or [T, heads*dim]), all float32.  The first C = 2*kv_heads*dim + heads*vdim columns of `proj` pass the
+    short causal convolution (conv_w [C, taps]; the inputs before the step come from conv_state [slots, taps-1, C], which
+    is then moved on), silu, and q and k become unit vectors per head (q times q_scale); beta = sigmoid(proj[:, col_b:]);
+    decay = exp(-exp(a_log) * softplus(a[:, col_a:] + dt_bias))."""
+    _need_cuda(proj, a, conv_w, a_log, dt_bias, conv_state, seq_of_token, slot_ids)
+    _rows2d("proj", proj)
+    _rows2d("a", a)
+    _need_i32("seq_of_token", seq_of_token)
+    _need_i32("slot_ids", slot_ids)
+    T = proj.shape[0]
+    C = 2 * kv_heads * dim + heads * vdim
+    per = dim if per_channel else 1
+    if proj.dtype != torch.float32 or a.dtype != torch.float32 or a.shape[0] != T or seq_of_token.numel() < T:
+        raise ValueError("delta_prepare takes float32 rows of projections, one per token")
+    if proj.shape[1] < max(C, col_b + heads) or col_b < 0 or col_a < 0 or a.shape[1] < col_a + heads * per:
+        raise ValueError("delta_prepare: the rows do not hold the columns asked for")
+    if conv_w.dim() != 2 or conv_w.shape[0] != C or not conv_w.is_contiguous() or not 1 <= conv_w.shape[1] <= DELTA_MAX_TAPS:
+        raise ValueError(f"the convolution's weights are contiguous [{C}, taps], taps at most {DELTA_MAX_TAPS}")
+    taps = conv_w.shape[1]
+    if (conv_state.dtype != torch.float32 or conv_state.dim() != 3 or tuple(conv_state.shape[1:]) != (max(taps - 1, 1), C)
+            or not conv_state.is_contiguous()):
+        raise ValueError(f"the convolution's state is contiguous float32 [slots, {max(taps - 1, 1)}, {C}]")
+    for name, t, n in (("a_log", a_log, heads), ("dt_bias", dt_bias, heads * per)):
+        if t.dtype != torch.float32 or tuple(t.shape) != (n,) or not t.is_contiguous():
+            raise ValueError(f"{name} is a contiguous float32 [{n}] tensor")
+    if C * 4 > 64 * 1024:
+        raise ValueError(f"{C} convolved channels do not fit one block's shared memory")
+    qkv = torch.empty(T, C, dtype=torch.float32, device=proj.device)
+    beta = torch.empty(T, heads, dtype=torch.float32, device=proj.device)
+    decay = torch.empty(T, heads * per, dtype=torch.float32, device=proj.device)
+    check(load().fmsamd_delta_prepare(proj.data_ptr(), proj.stride(0), col_b, a.data_ptr(), a.stride(0), col_a, conv_w.data_ptr(),
+                                      _code(conv_w.dtype), taps, a_log.data_ptr(), dt_bias.data_ptr(), conv_state.data_ptr(),
+                                      seq_of_token.data_ptr(), slot_ids.data_ptr(), qkv.data_ptr(), beta.data_ptr(), decay.data_ptr(),
+                                      T, heads, kv_heads, dim, vdim, int(bool(per_channel)), float(q_scale), _stream()))
+    return qkv, beta, decay
+
+
+def delta_rule(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, state: torch.Tensor, seq_starts: torch.Tensor,
+               seq_of_token: torch.Tensor, slot_ids: torch.Tensor, n_seqs: int, heads: int, kv_heads: int, dim: int, vdim: int,
+               per_channel: bool) -> torch.Tensor:
+    """The recurrence S = g S; u = beta (v - S^T k); S += k u^T; o = S^T q over the tokens of every sequence of the
+    step, from and into state [slots, heads, vdim, dim] (float32, S transposed) -> o float32 [T, heads*vdim].
+    Sequence b of the step owns the token rows seq_starts[b] .. seq_starts[b + 1] and the state of slot_ids[b]."""
+    _need_cuda(qkv, beta, decay, state, seq_starts, seq_of_token, slot_ids)
+    for name, t in (("seq_starts", seq_starts), ("seq_of_token", seq_of_token), ("slot_ids", slot_ids)):
+        _need_i32(name, t)
+    T = qkv.shape[0]
+    C = 2 * kv_heads * dim + heads * vdim
+    per = dim if per_channel else 1
+    for name, t, cols in (("qkv", qkv, C), ("beta", beta, heads), ("decay", decay, heads * per)):
+        if t.dtype != torch.float32 or tuple(t.shape) != (T, cols) or not t.is_contiguous():
+            raise ValueError(f"{name} is contiguous float32 [{T}, {cols}]")
+    if state.dtype != torch.float32 or state.dim() != 4 or tuple(state.shape[1:]) != (heads, vdim, dim) or not state.is_contiguous():
+        raise ValueError(f"the state is contiguous float32 [slots, {heads}, {vdim}, {dim}]")
+    if dim > DELTA_MAX_DIM:
+        raise ValueError(f"the delta rule keeps at most {DELTA_MAX_DIM} key channels a head, not {dim}")
+    if seq_starts.numel() < n_seqs + 1 or slot_ids.numel() < n_seqs or seq_of_token.numel() < T:
+        raise ValueError("the step's index arrays are shorter than its sequences or tokens")
+    out = torch.empty(T, heads * vdim, dtype=torch.float32, device=qkv.device)
+    check(load().fmsamd_delta_rule(qkv.data_ptr(), beta.data_ptr(), decay.data_ptr(), state.data_ptr(), out.data_ptr(),
+                                   seq_starts.data_ptr(), seq_of_token.data_ptr(), slot_ids.data_ptr(), n_seqs, heads, kv_heads, dim,
+                                   vdim, int(bool(per_channel)), _stream()))
+    return out
+
+
+def gated_head_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, activation: str, heads: int, vdim: int,
+                    out_dtype: torch.dtype, seq_of_token: torch.Tensor, scale: float = 1.0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """o float32 [T, heads*vdim]: every head divided by its root mean square, times weight [vdim], times act(gate)
+    (float32 logits [T, heads*vdim], rows of any stride), times scale -> out_dtype (into `out`, rows of any stride)."""
+    _need_cuda(o, gate, weight, seq_of_token, out)
+    _rows2d("gate", gate)
+    _need_i32("seq_of_token", seq_of_token)
+    T = o.shape[0]
+    if o.dtype != torch.float32 or tuple(o.shape) != (T, heads * vdim) or not o.is_contiguous():
+        raise ValueError(f"o is contiguous float32 [T, {heads * vdim}]")
+    if gate.dtype != torch.float32 or tuple(gate.shape) != (T, heads * vdim):
+        raise ValueError(f"the gate is float32 [{T}, {heads * vdim}]")
+    if tuple(weight.shape) != (vdim,) or not weight.is_contiguous():
+        raise ValueError(f"the norm weight is a contiguous [{vdim}] tensor")
+    if out is None:
+        out = torch.empty(T, heads * vdim, dtype=out_dtype, device=o.device)
+    _rows2d("out", out)
+    if out.dtype != out_dtype or tuple(out.shape) != (T, heads * vdim):
+        raise ValueError(f"out is [{T}, {heads * vdim}] of {out_dtype}")
+    check(load().fmsamd_gated_head_norm(o.data_ptr(), gate.data_ptr(), gate.stride(0), weight.data_ptr(), _code(weight.dtype), float(eps),
+                                        ACTIVATIONS[activation], float(scale), out.data_ptr(), _code(out_dtype), out.stride(0),
+                                        seq_of_token.data_ptr(), T, heads, vdim, _stream()))
     return out
 
 

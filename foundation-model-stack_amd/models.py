@@ -118,6 +118,8 @@ def get_model(
                 if arch.detect_source is None:
                     raise ValueError(f"architecture {arch.name} cannot tell a checkpoint's source from its tensor names: pass source=")
                 source = arch.detect_source(names)
+            if arch.sizes_from_tensors is not None:
+                config = arch.sizes_from_tensors(config, {n: ckpt.stored_shape(n) for n in names})
             floats = [ckpt.stored_dtype(n) for n in names if ckpt.stored_dtype(n).is_floating_point]
             if floats:
                 ckpt_dtype = torch.float32 if all(d in (torch.float32, torch.float64) for d in floats) else torch.bfloat16

@@ -41,7 +41,17 @@ class MultiHeadAttention(Mixer):
         scale_factor: Optional[float] = None,
         window: int = 0,
         soft_cap: float = 0.0,
+        value_dim: Optional[int] = None,
+        qkv_bias: Optional[bool] = None,
+        out_bias: Optional[bool] = None,
+        qk_norm: Optional[str] = None,
+        norm_eps: float = 1e-6,
+        output_gate: bool = False,
     ):
+        """value_dim: the size of a value (and of an output head) if it is not head_dim.  qkv_bias, out_bias: biases of the
+        input and the output projection (default: use_bias for both).  qk_norm "projection": queries and keys pass an RMS
+        norm over their whole projection (all heads at once, plain weights, norm_eps), before rotation.  output_gate: the
+        concatenated heads are multiplied by sigmoid(W_g h), h the mixer's input, before the output projection."""
         super().__init__()
         if kvheads <= 0 or nheads % kvheads:
             raise ValueError(f"{nheads} query heads are no multiple of {kvheads} kv heads")
@@ -54,18 +64,41 @@ class MultiHeadAttention(Mixer):
         if self.soft_cap < 0:
             raise ValueError(f"soft_cap {soft_cap} must be zero (none) or positive")
         self.position_encoder = position_encoder
+        self.value_dim = int(value_dim) if value_dim else head_dim
+        if not 0 < self.value_dim <= 256:
+            raise ValueError(f"value size {self.value_dim} must be at most 256")
+        if qk_norm not in (None, "projection"):
+            raise ValueError(f"qk_norm {qk_norm!r} is not one of None, 'projection'")
+        self.qk_norm, self.norm_eps, self.output_gate = qk_norm, float(norm_eps), bool(output_gate)
+        qkv_bias = use_bias if qkv_bias is None else bool(qkv_bias)
+        out_bias = use_bias if out_bias is None else bool(out_bias)
+        # the steps beyond Llama's attention run a path of their own; without them nothing changes
+        self.extended = bool(self.qk_norm or self.output_gate or self.value_dim != head_dim)
+        self.n_q, self.n_k, self.n_v = nheads * head_dim, kvheads * head_dim, kvheads * self.value_dim
         in_proj = self.add_child("in_proj", Part())
-        self.qkv = in_proj.add_child("qkv_fused", Linear(width, (nheads + 2 * kvheads) * head_dim, use_bias))
-        self.dense = self.add_child("dense", Linear(nheads * head_dim, width, use_bias))
+        # with an output gate the gate's rows follow the values: everything that reads the mixer's input is one product
+        rows = self.n_q + self.n_k + self.n_v + (nheads * self.value_dim if self.output_gate else 0)
+        self.qkv = in_proj.add_child("qkv_fused", Linear(width, rows, qkv_bias))
+        if self.qk_norm:
+            self.declare("q_norm.weight", (self.n_q,), init="ones", kind="scale")
+            self.declare("k_norm.weight", (self.n_k,), init="ones", kind="scale")
+        self.dense = self.add_child("dense", Linear(nheads * self.value_dim, width, out_bias))
 
     def unfused_parameters(self) -> dict:
         """The fused projection as the parts it is made of: fused local name -> ((local name, rows), ...), in the
         order of the rows (fms/modules/attention.py:666-687)."""
-        H, K, D = self.nheads, self.kvheads, self.head_dim
-        return {"in_proj.qkv_fused": (("in_proj.query", H * D), ("in_proj.key", K * D), ("in_proj.value", K * D))}
+        pieces = (("in_proj.query", self.n_q), ("in_proj.key", self.n_k), ("in_proj.value", self.n_v))
+        if self.output_gate:
+            pieces += (("in_proj.gate", self.nheads * self.value_dim),)
+        return {"in_proj.qkv_fused": pieces}
+
+    def output_projection(self) -> Linear:
+        return self.dense
 
     # ---- what the mixer asks of the cache ---------------------------------
     def kv_need(self) -> Optional[KVNeed]:
+        if self.value_dim != self.head_dim:
+            return KVNeed(self.kvheads, self.head_dim, self.window, value_dim=self.value_dim)
         return KVNeed(self.kvheads, self.head_dim, self.window)
 
     def state_need(self):
@@ -83,14 +116,15 @@ class MultiHeadAttention(Mixer):
         return self.position_encoder.score_slopes(self.nheads) if self.position_encoder is not None else None
 
     def prefill_qblock(self, n_tokens: int, dtype) -> int:
-        if dtype != torch.bfloat16 or self.head_dim % 16 or self.soft_cap > 0 or self._score_slopes() is not None:
+        if (dtype != torch.bfloat16 or self.head_dim % 16 or self.soft_cap > 0 or self._score_slopes() is not None
+                or self.value_dim != self.head_dim):
             return 0  # the generic kernel takes tokens one by one
         return ops.prefill_qblock(self.nheads, self.kvheads, self.head_dim, n_tokens)
 
     def _fused_decode(self, rows: int, dtype, batch) -> bool:
         """True if projection, rotation and cache write of this step run as one kernel."""
         rotates_by_table = self.position_encoder is None or self.position_encoder.rotary_tables() is not None
-        return (batch.is_decode and rows <= ops.QKV_ROPE_MAX_ROWS and dtype == torch.bfloat16
+        return (not self.extended and batch.is_decode and rows <= ops.QKV_ROPE_MAX_ROWS and dtype == torch.bfloat16
                 and self.qkv.w["weight"].dtype == torch.bfloat16 and self.head_dim % 16 == 0 and self.width % 8 == 0
                 and rotates_by_table)
 
@@ -100,7 +134,9 @@ class MultiHeadAttention(Mixer):
     def forward(self, x: torch.Tensor, batch, cache: LayerCache) -> torch.Tensor:
         return self.forward_branch(x, batch, cache).value()
 
-    def forward_branch(self, x, batch, cache: LayerCache) -> BranchOutput:
+    def forward_branch(self, x, batch, cache: LayerCache, out: Optional[torch.Tensor] = None, out_scale: float = 1.0) -> BranchOutput:
+        """out (rows [T, heads * value size] of any stride) and out_scale: where the input of the output projection is
+        written, and a factor on it, for a caller that runs this mixer beside another and projects both at once."""
         x, row_norm = split_normed(x)
         H, K, D = self.nheads, self.kvheads, self.head_dim
         table = batch.block_tables[cache.group]
@@ -108,7 +144,23 @@ class MultiHeadAttention(Mixer):
         cos, sin, rot = tables if tables is not None else (None, None, 0)
         keys, values = (cache.keys, cache.values) if cache.owns else (None, None)
         weight = self.qkv.w["weight"]
-        if self._fused_decode(x.shape[0], x.dtype, batch):
+        gate = None
+        if self.extended:
+            if row_norm is not None:
+                raise RuntimeError("a deferred norm reached a step that does not take one")
+            # norms and the gate are formed from the float32 sums of the projection
+            proj = self.qkv.forward(x, out_dtype=torch.float32)
+            if self.qk_norm:
+                qkv = ops.qk_projection_norm(proj, self.n_q, self.n_k, self.n_v, self.w["q_norm.weight"], self.w["k_norm.weight"],
+                                             self.norm_eps, x.dtype, batch.seq_of_token)
+            else:
+                qkv = ops.cast(proj[:, : self.n_q + self.n_k + self.n_v].contiguous(), x.dtype)
+            if self.output_gate:
+                gate = proj[:, self.n_q + self.n_k + self.n_v :]
+            if tables is None and self.position_encoder is not None:
+                self.position_encoder.adjust_qk(qkv, batch, H, K, D)
+            ops.rope_kv_write(qkv, batch.positions, batch.seq_of_token, table, cos, sin, rot, keys, values, H, K, D, self.value_dim)
+        elif self._fused_decode(x.shape[0], x.dtype, batch):
             # decode: projection, rotation and cache write in one kernel
             qkv = ops.qkv_rope_write(x, weight, self.qkv.w.get("bias"), batch.positions, batch.seq_of_token, table,
                                      cos, sin, rot, keys, values, H, K, D, row_norm=row_norm)
@@ -126,8 +178,10 @@ class MultiHeadAttention(Mixer):
             decode=batch.is_decode, max_context=batch.context_bound,
             qblock_start=qb_start, qblock_len=qb_len, qblock_tokens=size,
             row_order=batch.rows_by_length if batch.is_decode else None,
-            score_slopes=self._score_slopes(), soft_cap=self.soft_cap,
+            score_slopes=self._score_slopes(), soft_cap=self.soft_cap, value_dim=self.value_dim,
         )
+        if gate is not None or out is not None or out_scale != 1.0:
+            mixed = ops.gate_mul(mixed, gate, "sigmoid", out_scale, out=out)
         return BranchOutput(mixed, self.dense)
 
 

@@ -60,8 +60,8 @@ class ResidualStream:
             if (self.fuse_products and next_norm is not None and getattr(next_norm, "deferrable", lambda: False)()
                     and getattr(lin, "streams", lambda *a: False)(out.x.shape[0], out.x.dtype)
                     and self.resid.shape[1] == lin.out_features):
-                scaled, row_norm = ops.linear_into_stream(out.x, lin.w["weight"], lin.w.get("bias"), self.resid,
-                                                          next_norm.w.get("weight"), next_norm.eps)
+                scale = next_norm.scale_weight() if hasattr(next_norm, "scale_weight") else next_norm.w.get("weight")
+                scaled, row_norm = ops.linear_into_stream(out.x, lin.w["weight"], lin.w.get("bias"), self.resid, scale, next_norm.eps)
                 self.prepared = (next_norm, NormedRows(scaled, row_norm))
                 return
             out = out.value()
@@ -73,13 +73,16 @@ class PreNormBlock(Part):
     fuses_next_norm = True  # forward takes the norm that reads the stream after this block
     norm_arguments = ("norm1", "norm2")  # the norms the block is built with, by constructor argument
 
-    def __init__(self, mixer: Part, feed_forward: Part, norm1: Part, norm2: Part,
+    def __init__(self, mixer: Part, feed_forward: Optional[Part], norm1: Part, norm2: Part,
                  names=("ln", "attn", "ff_ln", "ff_sub_layer")):
+        """The feed-forward may be absent (None): the block is then its mixer branch alone, and has no second norm."""
         super().__init__()
         self.norm1 = self.add_child(names[0], norm1)
         self.mixer = self.add_child(names[1], mixer)
-        self.norm2 = self.add_child(names[2], norm2)
-        self.feed_forward = self.add_child(names[3], feed_forward)
+        self.feed_forward = feed_forward
+        if feed_forward is not None:
+            self.norm2 = self.add_child(names[2], norm2)
+            self.add_child(names[3], feed_forward)
 
     def first_norm(self) -> Part:
         return self.norm1
@@ -89,6 +92,9 @@ class PreNormBlock(Part):
         mixer_takes = getattr(self.mixer, "accepts_normed_rows", None)
         h = stream.normed(self.norm1, act_dtype, mixer_takes is not None and mixer_takes(T, act_dtype, batch))
         branch = getattr(self.mixer, "forward_branch", self.mixer.forward)
+        if self.feed_forward is None:
+            stream.add_branch(branch(h, batch, cache), next_norm)
+            return
         stream.add_branch(branch(h, batch, cache), self.norm2)
         ff_takes = getattr(self.feed_forward, "accepts_normed_rows", None)
         h = stream.normed(self.norm2, act_dtype, ff_takes is not None and ff_takes(T, act_dtype))

@@ -25,13 +25,14 @@ class TokenEmbedding(Part):
 
 
 class LinearHead(Part):
-    def __init__(self, width: int, vocab: int):
+    def __init__(self, width: int, vocab: int, scale: float = 1.0):
         super().__init__()
-        self.vocab, self.width = vocab, width
+        self.vocab, self.width, self.scale = vocab, width, float(scale)  # scale: a constant factor on every logit
         self.declare("weight", (vocab, width))
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return ops.linear(x, self.w["weight"], None, out_dtype=torch.float32)
+        logits = ops.linear(x, self.w["weight"], None, out_dtype=torch.float32)
+        return logits if self.scale == 1.0 else ops.scale_(logits, self.scale)
 
 
 register_part("embedding", "table", TokenEmbedding)

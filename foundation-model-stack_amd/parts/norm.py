@@ -24,13 +24,27 @@ class ParameterizedNorm(Part):
         elementwise_scale: bool = True,
         elementwise_shift: bool = False,
         use_mean: bool = False,
+        weight_offset: float = 0.0,
     ):
+        """weight_offset: the stored weight is the scale minus this number (1.0 for a scale stored around zero); the sum
+        is formed once, in float32, when the model is finalized."""
         super().__init__()
         self.width, self.eps, self.use_mean = width, float(eps), use_mean
+        self.weight_offset = float(weight_offset)
+        self._scale: Optional[torch.Tensor] = None
         if elementwise_scale:
-            self.declare("weight", (width,), init="ones", kind="scale")
+            # random-weights mode gives a scale of one either way
+            self.declare("weight", (width,), init="ones" if self.weight_offset == 0.0 else "zeros", kind="scale")
         if elementwise_shift:
             self.declare("bias", (width,), init="zeros", kind="scale")
+
+    def finalize(self, device, dtype) -> None:
+        if self.weight_offset and self.w.get("weight") is not None:
+            self._scale = (self.w["weight"].to(torch.float32) + self.weight_offset).contiguous()
+
+    def scale_weight(self) -> Optional[torch.Tensor]:
+        """The scale that multiplies the normed rows: the stored weight, plus its offset if it has one."""
+        return self._scale if self._scale is not None else self.w.get("weight")
 
     def add_norm(
         self,
@@ -46,9 +60,12 @@ class ParameterizedNorm(Part):
         if branch_norm is not None and branch is not None:
             if not (self.deferrable() and branch_norm.deferrable()):
                 raise NotImplementedError("a normed branch is added by RMS norms without mean and shift only")
-            return ops.norm_add_norm(resid, branch, branch_norm.w.get("weight"), branch_norm.eps, self.w.get("weight"), self.eps,
+            return ops.norm_add_norm(resid, branch, branch_norm.scale_weight(), branch_norm.eps, self.scale_weight(), self.eps,
                                      out_dtype, rows)
-        return ops.add_norm(resid, branch, self.w.get("weight"), self.w.get("bias"), self.eps, out_dtype, rows, self.use_mean)
+        bias = self.w.get("bias")
+        if bias is not None and self._scale is not None:
+            bias = bias.to(torch.float32)  # the kernel takes scale and shift of one type
+        return ops.add_norm(resid, branch, self.scale_weight(), bias, self.eps, out_dtype, rows, self.use_mean)
 
     def deferrable(self) -> bool:
         """True if the norm is a row scale times a weight (no mean, no shift), so that a product can apply the

@@ -45,12 +45,13 @@ def rope_frequencies(dim: int, theta: float, scaling: Optional[dict] = None, alp
     if kind == "ntk":
         theta = theta * alpha ** (dim / (dim - 2))
     if exact:
-        # theta^(-2i/dim) formed in float64 and rounded once, for models that define the frequencies as real numbers
-        freqs = torch.tensor([float(theta) ** (-2.0 * i / dim) for i in range(dim // 2)], dtype=torch.float64).to(torch.float32)
+        # theta^(-2i/dim) formed in float64 and rounded once at the end (after any scaling), for models that define the
+        # frequencies as real numbers
+        freqs = torch.tensor([float(theta) ** (-2.0 * i / dim) for i in range(dim // 2)], dtype=torch.float64)
     else:
         freqs = 1.0 / (theta ** (torch.arange(0, dim, 2)[: dim // 2].float() / dim))
     if kind in ("regular", "ntk"):
-        return freqs
+        return freqs.to(torch.float32)
     if kind == "llama3":
         factor = scaling["factor"]
         low_freq_factor = scaling["low_freq_factor"]
@@ -61,7 +62,7 @@ def rope_frequencies(dim: int, theta: float, scaling: Optional[dict] = None, alp
         smooth = (old_len / wavelen - low_freq_factor) / (high_freq_factor - low_freq_factor)
         smoothed = (1 - smooth) * scaled / factor + smooth * scaled
         medium = ~(wavelen < old_len / high_freq_factor) * ~(wavelen > old_len / low_freq_factor)
-        return torch.where(medium, smoothed, scaled)
+        return torch.where(medium, smoothed, scaled).to(torch.float32)
     raise ValueError(f"rope_type {kind!r} is not supported (regular, llama3, ntk)")
 
 
@@ -93,11 +94,14 @@ class RotaryEncoding(PositionEncoding):
     the encoding is the regular one (tests/modules/test_positions.py:216-241)."""
 
     def __init__(self, dim: int, theta: float = 10_000.0, max_seq_len: int = 2048, scaling: Optional[dict] = None,
-                 partial_rope: float = 1.0, max_positions: Optional[int] = None, exact_frequencies: bool = False):
+                 partial_rope: float = 1.0, max_positions: Optional[int] = None, exact_frequencies: bool = False,
+                 rot_dim: Optional[int] = None):
+        """rot_dim: the number of rotated dimensions of a head, for a model that gives it as a number (default:
+        partial_rope times the head size)."""
         super().__init__()
         self.exact_frequencies = bool(exact_frequencies)
         self.head_dim = dim
-        self.rot_dim = int(partial_rope * dim)
+        self.rot_dim = int(rot_dim) if rot_dim is not None else int(partial_rope * dim)
         if self.rot_dim % 2 or self.rot_dim <= 0 or self.rot_dim > dim:
             raise ValueError(f"rotary size {self.rot_dim} of head size {dim} must be even and within the head")
         self.theta, self.max_seq_len, self.scaling = float(theta), int(max_seq_len), dict(scaling or {})
