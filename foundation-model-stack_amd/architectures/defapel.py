@@ -217,7 +217,7 @@ register_architecture(
 def make_config(width: int, vocab: int, pattern: str, heads: int, kv_heads: int, dim: int, vdim: int, window: int, delta_heads: int,
                 delta_kv_heads: int, delta_dim: int, delta_vdim: int, experts: int, top: int, expert_ff: int, conv: int = 4,
                 rot_dims: int = 0, rot_base: float = 500000.0, rot_scaling: dict = None, softcap: float = 30.0, rank: int = 0,
-                left_scale: float = 1.0, right_scale: float = 1.0, logit_scale: float = 1.0, max_positions: int = 32768) -> DefapelConfig:
+                left_scale: float = 1.0, right_scale: float = 1.0, logit_scale: float = 1.0, max_positions: int = 131072) -> DefapelConfig:
     """A regular Defapel: `pattern` has a letter per layer, "p" for a parallel mixer and "c" for a channel_delta one; all
     layers of a kind share their sizes."""
     layers = []

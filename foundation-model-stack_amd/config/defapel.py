@@ -31,7 +31,7 @@ class DefapelConfig(ModelConfig):
     layers: List[dict] = dataclasses.field(default_factory=list)
     norm: dict = dataclasses.field(default_factory=lambda: {"eps": 1e-6})
     logit_scale: float = 1.0
-    max_positions: int = 32768
+    max_positions: int = 131072
 
     def __post_init__(self):
         self.validate()

@@ -18,8 +18,9 @@ import torch
 # What a product's or an activation's result is stored as.  Identity for the exact run; a round trip through bfloat16
 # for the run that shows what bfloat16 storage costs (what the design computes in 32-bit stays as it is).
 _store = lambda x: x  # noqa: E731
-# When a list: every mixture-of-experts layer appends, per token, by how much the last chosen expert's score exceeds
-# the best score not chosen (inf when all experts are chosen).
+# When a list: every mixture-of-experts layer appends, per token, by how much the last chosen expert's router logit
+# exceeds the best logit not chosen (inf when all experts are chosen).  A small number marks a choice that rounding
+# can turn: such a token's logits are no test of arithmetic.
 router_margins = None
 
 
@@ -174,11 +175,12 @@ def gated_delta(h, w, p, m, eps, per_channel):
 def experts(h, w, p, mlp):
     """Every token's `top` experts by sigmoid score; the score scales the expert's input."""
     E, top = mlp["router"]["experts"], mlp["router"]["top"]
-    scores = torch.sigmoid(h @ w[p + "router"].T)
+    z = h @ w[p + "router"].T
+    scores = torch.sigmoid(z)
     best, ids = torch.topk(scores, top, dim=-1)
     if router_margins is not None:
-        rest = scores.scatter(1, ids, float("-inf")).max(dim=-1).values if top < E else torch.full((h.shape[0],), float("-inf"))
-        router_margins.append(best[:, -1] - rest)
+        rest = z.scatter(1, ids, float("-inf")).max(dim=-1).values if top < E else torch.full((h.shape[0],), float("-inf"))
+        router_margins.append(z.gather(1, ids).min(dim=-1).values - rest)
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for s, e in zip(best[t], ids[t]):
@@ -222,3 +224,11 @@ def forward(config, w, tokens, rounding=None, return_layers=False):
         return (logits, torch.stack(layers)) if return_layers else logits
     finally:
         _store = lambda x: x  # noqa: E731
+
+
+def greedy_generate(config, w, prompt, n_new):
+    """The n_new tokens that greedy decoding appends to `prompt` (the whole sequence is run again for every token)."""
+    ids = list(prompt)
+    for _ in range(n_new):
+        ids.append(int(torch.argmax(forward(config, w, ids)[-1])))
+    return ids[len(prompt):]
