@@ -17,6 +17,11 @@ is another workload (the default one and its record stay as they are): Zodolorn 
 Llama models of the same width, depth, heads and feed-forward parameters: prefill and decode throughput of both, and
 for every class of kernel its time in one eager prefill and one eager decode step over the time that its bytes and
 flops would take at what this GPU delivers (`x_roofline`: 1 is the roofline).
+
+    python bench.py --defapel [--layers N]
+
+is the same comparison for Defapel (windowed attention beside a gated delta rule, a delta rule with a decay per channel,
+experts weighted on their input) beside Llama of the same width, depth and heads.
 """
 
 import argparse
@@ -60,6 +65,7 @@ def main() -> int:
     ap.add_argument("--max_new_tokens", type=int, default=None, help="the same as --steps: decode steps that are timed")
     ap.add_argument("--zodolorn", action="store_true",
                     help="another workload: Zodolorn beside Llama at equal layer sizes, with every kernel class's distance from its roofline")
+    ap.add_argument("--defapel", action="store_true", help="another workload: Defapel beside Llama at equal layer sizes, likewise")
     args = ap.parse_args()
     if args.seq_len is not None:
         args.prompt_min = args.prompt_max = args.seq_len
@@ -71,8 +77,8 @@ def main() -> int:
         print(f"bench.py measures one GPU: this library runs on a single MI355X, --gpus {args.gpus} is not supported")
         return 2
 
-    if args.zodolorn:
-        return zodolorn_comparison(args)
+    if args.zodolorn or args.defapel:
+        return design_comparison(args, "zodolorn" if args.zodolorn else "defapel")
 
     import torch
 
@@ -306,7 +312,15 @@ ZODOLORN_SIZES = [
 ]
 
 
-def zodolorn_comparison(args) -> int:
+# (name, width, layer pattern, heads, kv heads, head size, window, delta heads, delta q/k heads, key channels, value channels,
+#  experts, top, expert ff, vocabulary)
+DEFAPEL_SIZES = [
+    ("w2048", 2048, "pppc", 16, 4, 128, 1024, 16, 8, 128, 128, 32, 4, 1024, 32768),
+    ("w4096", 4096, "pppc", 32, 8, 128, 1024, 32, 16, 128, 128, 64, 6, 1536, 32768),
+]
+
+
+def design_comparison(args, design) -> int:
     import torch
 
     import fms_amd
@@ -339,6 +353,11 @@ def zodolorn_comparison(args) -> int:
         if name == "attention":  # grouped-query attention over keys and values of kvheads x head_dim
             H, K, D = a[6], a[7], a[8]
             return 2 * state["keys_loaded"] * 2 * K * D + 2 * nbytes(a[0][:, : H * D]), 4.0 * state["keys_read"] * H * D
+        if name == "delta_rule":  # state read and written once a sequence; per token and head 4 passes over dim x vdim in float32
+            qkv, st, n_seqs, H, D, V = a[0], a[4], a[8], a[9], a[11], a[12]
+            vector_flops = 8.0 * qkv.shape[0] * H * D * V
+            # priced at the float32 vector rate (the recurrence runs there), in units of the matrix rate the ideal is formed with
+            return nbytes(qkv, a[1], a[2], out) + 2 * n_seqs * (st.numel() // st.shape[0]) * 4, vector_flops * mfma_flops / PEAK_FLOPS["fp32"]
         if name == "latent_attention":  # one row of rank + rot a key, and the latent once more as values
             H, R, P = a[6], a[7], a[8]
             return 2 * state["keys_loaded"] * (2 * R + P) + nbytes(a[0]) + 2 * a[0].shape[0] * H * R, 2.0 * state["keys_read"] * H * (2 * R + P)
@@ -351,9 +370,11 @@ def zodolorn_comparison(args) -> int:
 
     watched = ["linear", "gated_linear", "linear_into_stream", "headwise_linear", "attention", "latent_attention", "moe_experts",
                "moe_route", "moe_combine", "add_norm", "norm_add_norm", "rms_norm_cols", "rope_kv_write", "qkv_rope_write",
-               "latent_kv_write", "latent_q_rotate", "activation", "clamped_gated_act", "gated_act", "embed"]
+               "latent_kv_write", "latent_q_rotate", "activation", "clamped_gated_act", "gated_act", "embed",
+               "delta_rule", "delta_prepare", "gated_head_norm", "qk_projection_norm", "gate_mul", "scale_", "cast"]
     small = {"moe_route", "moe_combine", "add_norm", "norm_add_norm", "rms_norm_cols", "rope_kv_write", "latent_kv_write",
-             "latent_q_rotate", "activation", "clamped_gated_act", "gated_act", "embed"}
+             "latent_q_rotate", "activation", "clamped_gated_act", "gated_act", "embed", "delta_prepare", "gated_head_norm",
+             "qk_projection_norm", "gate_mul", "scale_", "cast"}
 
     def classes_of_a_step(run):
         """{class: (ms, ms at the roofline)} of the kernels of `run()`, by events around every call into the library."""
@@ -385,7 +406,11 @@ def zodolorn_comparison(args) -> int:
             out[kind] = (ms + first.elapsed_time(last), ideal + 1000 * max(b / read_bps, f / mfma_flops))
         return {k: {"ms": round(ms, 4), "x_roofline": round(ms / ideal, 2) if ideal else None} for k, (ms, ideal) in sorted(out.items())}
 
-    def measure(model, vocab):
+    def measure(model, vocab, window=0):
+        """window: the most keys a query of the model's attention sees (0: all before it), for the attention's flops."""
+        def keys_seen(lengths):
+            return sum(min(n, window) if window else n for n in lengths)
+
         out = {}
         for n in (512, 2048):
             engine = Engine(model, max_tokens=n + 64, max_slots=1, use_graphs=False)
@@ -404,7 +429,7 @@ def zodolorn_comparison(args) -> int:
             out[f"prefill_{n}_ms"] = round(1000 * t, 3)
             if n == 2048:
                 slot = engine.new_sequence()
-                state.update(keys_read=n * (n + 1) // 2, keys_loaded=n)
+                state.update(keys_read=keys_seen(range(1, n + 1)), keys_loaded=n)
                 out["prefill_2048_kernels"] = classes_of_a_step(lambda: engine.step([slot], [ids], "last"))
                 engine.end_sequence(slot)
             del engine
@@ -437,7 +462,8 @@ def zodolorn_comparison(args) -> int:
             out[f"{name}_tok_s"] = round(batch * steps / dt, 1)
             out[f"{name}_ms"] = round(1000 * dt / steps, 3)
             if (batch, prompt) in ((8, 1024), (8, 7000)):
-                state.update(keys_read=sum(lens) + batch * (warmup + steps + 1), keys_loaded=sum(lens) + batch * (warmup + steps + 1))
+                now = [n + warmup + steps + 1 for n in lens]
+                state.update(keys_read=keys_seen(now), keys_loaded=keys_seen(now))
                 out[f"{name}_kernels"] = classes_of_a_step(lambda: engine.step(slots, [[t] for t in tokens], "last"))
             for s in slots:
                 engine.end_sequence(s)
@@ -445,9 +471,35 @@ def zodolorn_comparison(args) -> int:
             torch.cuda.empty_cache()
         return out
 
-    record = {"workload": "zodolorn beside llama at equal layer sizes", "layers": layers, "dtype": "bf16",
+    record = {"workload": f"{design} beside llama at equal layer sizes", "layers": layers, "dtype": "bf16",
               "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
               "peak_measured": {"read_gbs": round(read_bps / 1e9, 1), "mfma_tflops": round(mfma_flops / 1e12, 1)}, "sizes": {}}
+    if design == "defapel":
+        from fms_amd.architectures.defapel import make_config as make_defapel
+
+        for name, width, pattern, heads, kv, dim, window, dheads, dkv, ddim, dvdim, experts, top, expert_ff, vocab in DEFAPEL_SIZES:
+            pattern = (pattern * layers)[:layers]
+            config = make_defapel(width=width, vocab=vocab, pattern=pattern, heads=heads, kv_heads=kv, dim=dim, vdim=dim, window=window,
+                                  delta_heads=dheads, delta_kv_heads=dkv, delta_dim=ddim, delta_vdim=dvdim, experts=experts, top=top,
+                                  expert_ff=expert_ff, max_positions=context)
+            model = fms_amd.from_config(config, "defapel", data_type="bf16", random_seed=args.seed)
+            mine = measure(model, vocab, window=window)
+            del model
+            torch.cuda.empty_cache()
+            # Llama of the same width, depth and heads; its gated feed-forward has the parameters of the experts a token uses
+            hidden = top * expert_ff
+            llama = fms_amd.get_model("llama", "micro", data_type="bf16", random_seed=args.seed, emb_dim=width, nheads=heads, kvheads=kv,
+                                      nlayers=layers, hidden_dim=hidden, src_vocab_size=vocab, max_expected_seq_len=context)
+            theirs = measure(llama, vocab)
+            del llama
+            torch.cuda.empty_cache()
+            record["sizes"][name] = {"defapel": dict(config=dict(width=width, pattern=pattern, heads=heads, kv_heads=kv, dim=dim, window=window,
+                                                                   delta_heads=dheads, delta_kv_heads=dkv, delta_dim=ddim, delta_vdim=dvdim,
+                                                                   experts=experts, top=top, expert_ff=expert_ff, vocab=vocab), **mine),
+                                     "llama": dict(config=dict(width=width, heads=heads, kvheads=kv, head_dim=width // heads, hidden=hidden,
+                                                               vocab=vocab), **theirs)}
+        print(json.dumps(record))
+        return 0
     for name, width, heads, (dim, rot, vdim, q_rank, kv_rank), dense_ff, experts, top, expert_ff, shared_ff, vocab in ZODOLORN_SIZES:
         config = make_config(width=width, vocab=vocab, nlayers=layers, heads=heads, dim=dim, rot_dim=rot, vdim=vdim, q_rank=q_rank,
                              kv_rank=kv_rank, dense_ff=dense_ff, experts=experts, top=top, expert_ff=expert_ff, shared_ff=shared_ff,

@@ -93,6 +93,23 @@ __global__ void __launch_bounds__(GEN_THREADS)
 }
 
 #define LOG2E 1.4426950408889634f
+
+// What turns a raw score q . k into the exponent of its probability: scale2 = softmax scale * log2(e), and, for capped
+// scores (score = cap * tanh(scale * q . k / cap)), the two factors of a transformation of the raw score that leaves the
+// rest of the softmax as it is: raw' = cap_out * tanh(raw * cap_in), cap_in = scale / cap, cap_out = cap / scale.
+// cap_in 0: no cap (a uniform branch that costs nothing).
+struct Scale2 {
+  float v, cap_in, cap_out;
+  __device__ __forceinline__ operator float() const { return v; }
+};
+__device__ __forceinline__ Scale2 make_scale2(float scale, float soft_cap) {
+  return Scale2{scale * LOG2E, soft_cap > 0.f ? scale / soft_cap : 0.f, soft_cap > 0.f ? soft_cap / scale : 0.f};
+}
+// tanh from the hardware's exponential and reciprocal: 1 - 2 / (1 + e^(2x)); exact at both ends (e^(2x) = inf or 0)
+__device__ __forceinline__ float capped(float raw, Scale2 s) {
+  const float e = __builtin_amdgcn_exp2f(raw * (s.cap_in * 2.f * LOG2E));
+  return s.cap_out * (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + e));
+}
 // the maximum that a partial result of the decode kernel carries when it holds no key at all
 #define DECODE_EMPTY -1e30f
 
@@ -183,13 +200,17 @@ __device__ __forceinline__ void step_scores(f32x4 (&sa)[QT], f32x4 (&sb)[QT], co
 template <int MAXDT, int QT>
 __device__ __forceinline__ void step_softmax(WaveState<MAXDT, QT>& st, f32x4 (&sa)[QT], f32x4 (&sb)[QT],
                                              bf16x8 (&pmat)[QT], const int (&qpos)[QT], const int (&qlo)[QT], int key0,
-                                             int head_dim, float scale2, bool full) {
+                                             int head_dim, Scale2 scale2, bool full) {
   const int g = (threadIdx.x & (WAVE - 1)) >> 4;
   const int ndt = head_dim / 16;
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
     // maxima of the raw scores, scaled once (the scale is positive); every probability is then one fused
     // multiply-add and one exponential: exp2(s * scale2 - m)
+    if (scale2.cap_in != 0.f) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sa[qt][i] = capped(sa[qt][i], scale2), sb[qt][i] = capped(sb[qt][i], scale2);
+    }
     if (!full) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -245,7 +266,7 @@ __device__ __forceinline__ void step_accumulate(WaveState<MAXDT, QT>& st, const 
 template <int MAXDT, int QT>
 __device__ __forceinline__ void half_step(WaveState<MAXDT, QT>& st, const bf16x8 (&qreg)[QT][(MAXDT + 1) / 2],
                                           const int (&qpos)[QT], const int (&qlo)[QT], int key0, const bf16* kbase,
-                                          int k_stride, const bf16* vbase, int v_stride, int head_dim, float scale2,
+                                          int k_stride, const bf16* vbase, int v_stride, int head_dim, Scale2 scale2,
                                           bool full) {
   f32x4 sa[QT], sb[QT];
   bf16x8 pmat[QT];
@@ -260,7 +281,7 @@ __device__ __forceinline__ void attn_wave_pages(WaveState<MAXDT, QT>& st, const 
                                                 const int (&qpos)[QT], const int (&qlo)[QT], int key_lo, int key_hi,
                                                 int page_first, int page_step, const int* __restrict__ bt,
                                                 const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
-                                                size_t page_elems, int kh, int head_dim, float scale, int full_lo,
+                                                size_t page_elems, int kh, int head_dim, Scale2 scale2, int full_lo,
                                                 int full_hi) {
   // full_lo..full_hi: the keys that every column of the wave sees (no mask needed inside)
   if (key_hi < key_lo) return;
@@ -274,7 +295,7 @@ __device__ __forceinline__ void attn_wave_pages(WaveState<MAXDT, QT>& st, const 
       const int key0 = pi * PAGE_TOKENS + half * 32;
       if (key0 > key_hi || key0 + 31 < key_lo) continue;  // uniform over the wave
       half_step<MAXDT, QT>(st, qreg, qpos, qlo, key0, kp + (size_t)half * 32 * head_dim, head_dim, vp + half * 32,
-                           PAGE_TOKENS, head_dim, scale * LOG2E, key0 + 31 <= full_hi && key0 >= full_lo);
+                           PAGE_TOKENS, head_dim, scale2, key0 + 31 <= full_hi && key0 >= full_lo);
     }
   }
 }
@@ -318,7 +339,7 @@ __global__ void __launch_bounds__(WAVES* WAVE)
                              const int* __restrict__ qblock_start, const int* __restrict__ qblock_len,
                              const int* __restrict__ block_table, int table_stride, const bf16* __restrict__ k_cache,
                              const bf16* __restrict__ v_cache, int nheads, int kvheads, int head_dim, float scale,
-                             int window) {
+                             int window, float soft_cap) {
   static_assert(WAVES * QT * 16 == PREFILL_QBLOCK, "a block covers PREFILL_QBLOCK tokens");
   const int h = blockIdx.y;
   const int wave = threadIdx.x / WAVE;
@@ -360,7 +381,7 @@ __global__ void __launch_bounds__(WAVES* WAVE)
   const int full_hi = positions[t0];
   const int full_lo = (window > 0 && key_hi - window + 1 > 0) ? key_hi - window + 1 : 0;
   attn_wave_pages<MAXDT, QT>(st, qreg, qpos, qlo, key_lo, key_hi, key_lo / PAGE_TOKENS, 1, bt, k_cache, v_cache,
-                             page_elems, kh, head_dim, scale, full_lo, full_hi);
+                             page_elems, kh, head_dim, make_scale2(scale, soft_cap), full_lo, full_hi);
 
   const int ndt = head_dim / 16;
 #pragma unroll
@@ -404,7 +425,7 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
                             const int* __restrict__ qblock_start, const int* __restrict__ qblock_len,
                             int n_qblocks, const int* __restrict__ block_table, int table_stride,
                             const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache, int nheads,
-                            int kvheads, int head_dim_arg, float scale, int window, int hb) {
+                            int kvheads, int head_dim_arg, float scale, int window, int hb, float soft_cap) {
   const int head_dim = EXACT ? MAXDT * 16 : head_dim_arg;
   constexpr int KS = MAXDT * 16 + LDS_PAD;    // LDS row stride of the key page [64][KS]
   constexpr int VS = PAGE_TOKENS + LDS_PAD;   // LDS row stride of the transposed value page [head_dim][VS]
@@ -521,7 +542,7 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
       const int key0 = pi * PAGE_TOKENS + khalf * 32;
       if (has_work && pi <= page_last && !(key0 > wave_hi || key0 + 31 < wave_lo))  // uniform over the wave
         half_step<MAXDT, QT>(st, qreg, qpos, qlo, key0, ks + cur * PAGE_ELEMS + khalf * 32 * KS, KS,
-                             vs + cur * PAGE_ELEMS + khalf * 32, VS, head_dim, scale * LOG2E,
+                             vs + cur * PAGE_ELEMS + khalf * 32, VS, head_dim, make_scale2(scale, soft_cap),
                              key0 + 31 <= full_hi && key0 >= full_lo);
       block_sync_lds();  // the page just multiplied is overwritten after the next one
     }
@@ -590,7 +611,7 @@ struct WaveState32 {
 template <int DT32>
 __device__ __forceinline__ void half_step32(WaveState32<DT32>& st, const bf16x8 (&qreg)[DT32 * 2], int qpos, int qlo,
                                             int key0, const bf16* kbase, int k_stride, const bf16* vbase, int v_stride,
-                                            float scale2, bool full) {
+                                            Scale2 scale2, bool full) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int j = lane & 31, hb = lane >> 5;
   // the key of tile row i = lane % 32 (this lane's row of the A operand): i = 8 blk + 4 h + e
@@ -604,6 +625,10 @@ __device__ __forceinline__ void half_step32(WaveState32<DT32>& st, const bf16x8 
     for (int c = 0; c < DT32 * 2; ++c) ka[c] = load_bf16x8(kbase + (size_t)key_row * k_stride + c * 16 + hb * 8);
 #pragma unroll
     for (int c = 0; c < DT32 * 2; ++c) sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[c], qreg[c], sc, 0, 0, 0);
+  }
+  if (scale2.cap_in != 0.f) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) sc[v] = capped(sc[v], scale2);
   }
   if (!full) {
 #pragma unroll
@@ -655,7 +680,7 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
                               const int* __restrict__ qblock_start, const int* __restrict__ qblock_len,
                               int n_qblocks, const int* __restrict__ block_table, int table_stride,
                               const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache, int nheads,
-                              int kvheads, float scale, int window, int hb) {
+                              int kvheads, float scale, int window, int hb, float soft_cap) {
   constexpr int head_dim = DT32 * 32;
   constexpr int KS = head_dim + LDS_PAD;      // LDS row stride of the key page [64][KS]
   constexpr int VS = PAGE_TOKENS + LDS_PAD;   // LDS row stride of the transposed value page [head_dim][VS]
@@ -766,7 +791,7 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
       const int key0 = pi * PAGE_TOKENS + khalf * 32;
       if (has_work && pi <= page_last && !(key0 > wave_hi || key0 + 31 < wave_lo))  // uniform over the wave
         half_step32<DT32>(st, qreg, qpos, qlo, key0, ks + cur * PAGE_ELEMS + khalf * 32 * KS, KS,
-                          vs + cur * PAGE_ELEMS + khalf * 32, VS, scale * LOG2E, key0 + 31 <= full_hi && key0 >= full_lo);
+                          vs + cur * PAGE_ELEMS + khalf * 32, VS, make_scale2(scale, soft_cap), key0 + 31 <= full_hi && key0 >= full_lo);
       block_sync_lds();  // the page just multiplied is overwritten after the next one
     }
   }
@@ -820,7 +845,7 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
 template <int MAXDT, int HALVES>
 __device__ __forceinline__ void decode_math(WaveState<MAXDT, 1>& st, const bf16x8 (&qreg)[(MAXDT + 1) / 2], int qpos,
                                             int qlo, int key0, const bf16x8 (&kreg)[HALVES][2][(MAXDT + 1) / 2],
-                                            const bf16x8 (&vreg)[HALVES][MAXDT], int head_dim, float scale2) {
+                                            const bf16x8 (&vreg)[HALVES][MAXDT], int head_dim, Scale2 scale2) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int g = lane >> 4;
   const int ndt = head_dim / 16;
@@ -835,6 +860,10 @@ __device__ __forceinline__ void decode_math(WaveState<MAXDT, 1>& st, const bf16x
         sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[hf][0][c], qreg[c], sa, 0, 0, 0);
         sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[hf][1][c], qreg[c], sb, 0, 0, 0);
       }
+    }
+    if (scale2.cap_in != 0.f) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sa[i] = capped(sa[i], scale2), sb[i] = capped(sb[i], scale2);
     }
     if (!(k0 + 31 <= qpos && k0 >= qlo)) {  // uniform: not all 32 keys are visible
 #pragma unroll
@@ -875,7 +904,7 @@ __device__ __forceinline__ void decode_math(WaveState<MAXDT, 1>& st, const bf16x
 template <int MAXDT, int HALVES>
 __device__ __forceinline__ void decode_keys(WaveState<MAXDT, 1>& st, const bf16x8 (&qreg)[(MAXDT + 1) / 2], int qpos,
                                             int qlo, int key0, const bf16* __restrict__ kp,
-                                            const bf16* __restrict__ vp, int head_dim, float scale2) {
+                                            const bf16* __restrict__ vp, int head_dim, Scale2 scale2) {
   // HALVES halves of 32 keys starting at key0 (kp/vp point at the page, `first` is the half inside it)
   const int lane = threadIdx.x & (WAVE - 1);
   const int r = lane & 15;
@@ -930,7 +959,7 @@ __device__ __forceinline__ void staged_load(bf16x8 (&raw)[16], const bf16* __res
 template <bool PREFETCH>
 __device__ __forceinline__ void staged_page_step(WaveState<8, 1>& st, const bf16x8 (&qreg)[4], int qpos, int qlo,
                                                  int key0, bf16x8 (&raw)[16], const bf16* __restrict__ vp,
-                                                 const bf16* __restrict__ kn, bf16* __restrict__ buf, float scale2) {
+                                                 const bf16* __restrict__ kn, bf16* __restrict__ buf, Scale2 scale2) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int r = lane & 15;
   const int g = lane >> 4;
@@ -967,6 +996,12 @@ __device__ __forceinline__ void staged_page_step(WaveState<8, 1>& st, const bf16
     }
   }
 
+  if (scale2.cap_in != 0.f) {
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sa[hf][i] = capped(sa[hf][i], scale2), sb[hf][i] = capped(sb[hf][i], scale2);
+  }
   if (!(key0 + PAGE_TOKENS - 1 <= qpos && key0 >= qlo)) {  // uniform: not all 64 keys are visible
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf)
@@ -1036,7 +1071,7 @@ __device__ __forceinline__ void staged_page_step(WaveState<8, 1>& st, const bf16
 __device__ __forceinline__ void decode_pages_staged(WaveState<8, 1>& st, const bf16x8 (&qreg)[4], int qpos, int qlo,
                                                     int first, int stride, int last, const int* __restrict__ bt,
                                                     const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
-                                                    size_t page_elems, int kh, bf16* __restrict__ buf, float scale2) {
+                                                    size_t page_elems, int kh, bf16* __restrict__ buf, Scale2 scale2) {
   if (first > last) return;
   const size_t head_off = (size_t)kh * PAGE_TOKENS * 128;
   bf16x8 raw[16];
@@ -1077,7 +1112,7 @@ __global__ void __launch_bounds__(MAXW* WAVE) __attribute__((amdgpu_waves_per_eu
                             const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                             const int* __restrict__ block_table, int table_stride, const bf16* __restrict__ k_cache,
                             const bf16* __restrict__ v_cache, int nheads, int kvheads, int head_dim, float scale,
-                            int window, int tile_cols, const int* __restrict__ row_order) {
+                            int window, int tile_cols, const int* __restrict__ row_order, float soft_cap) {
   extern __shared__ float lds_dynamic[];  // not staged: [wave][tile_cols columns][head_dim + 2]
   __shared__ __attribute__((aligned(16))) bf16 stage[STAGED ? MAXW * 8192 : 8];
   // where the waves' partial results meet: a region of its own, or (staged) the head of each wave's page buffer
@@ -1133,17 +1168,17 @@ __global__ void __launch_bounds__(MAXW* WAVE) __attribute__((amdgpu_waves_per_eu
   if (STAGED) {
     if constexpr (MAXDT == 8)
       decode_pages_staged(st, qreg, pos, lo, page_lo + wave, n_waves, page_hi, bt, k_cache, v_cache, page_elems, kh,
-                          stage + wave * 8192, scale * LOG2E);
+                          stage + wave * 8192, make_scale2(scale, soft_cap));
   } else {
     for (int pi = page_lo + wave; pi <= page_hi; pi += n_waves) {
       const size_t phys = readable_page(uniform_load(bt + pi));
       const bf16* kp = k_cache + phys * page_elems + (size_t)kh * PAGE_TOKENS * head_dim;
       const bf16* vp = v_cache + phys * page_elems + (size_t)kh * head_dim * PAGE_TOKENS;
       if (MAXDT <= 8) {
-        decode_keys<MAXDT, 2>(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, head_dim, scale * LOG2E);
+        decode_keys<MAXDT, 2>(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, head_dim, make_scale2(scale, soft_cap));
       } else {  // large heads: half a page at a time keeps the loads in registers
-        decode_keys<MAXDT, 1>(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, head_dim, scale * LOG2E);
-        decode_keys<MAXDT, 1>(st, qreg, pos, lo, pi * PAGE_TOKENS + 32, kp, vp, head_dim, scale * LOG2E);
+        decode_keys<MAXDT, 1>(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, head_dim, make_scale2(scale, soft_cap));
+        decode_keys<MAXDT, 1>(st, qreg, pos, lo, pi * PAGE_TOKENS + 32, kp, vp, head_dim, make_scale2(scale, soft_cap));
       }
     }
   }
@@ -1312,7 +1347,7 @@ extern "C" int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out,
                                         const int* qblock_len, int n_qblocks, int qblock_tokens,
                                         const int* block_table, int table_stride, const void* k_cache,
                                         const void* v_cache, int n_tokens, int nheads, int kvheads, int head_dim,
-                                        float scale, int window, hipStream_t stream) {
+                                        float scale, int window, float soft_cap, hipStream_t stream) {
   if (n_tokens == 0 || n_qblocks == 0) return 0;
   if (check_common("attn_prefill_bf16", n_tokens, nheads, kvheads, head_dim, q_stride, out_stride)) return -1;
   FMS_REQUIRE(head_dim % 16 == 0, "attn_prefill_bf16: head size %d is no multiple of 16", head_dim);
@@ -1325,7 +1360,7 @@ extern "C" int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out,
     dim3 grid(n_qblocks, nheads);
     attn_prefill_bf16_kernel<16, 1, 8><<<grid, dim3(8 * WAVE), 0, stream>>>(
         (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, qblock_start, qblock_len,
-        block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, scale, window);
+        block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, scale, window, soft_cap);
     FMS_LAUNCH_CHECK("attn_prefill_bf16");
     return 0;
   }
@@ -1342,17 +1377,17 @@ extern "C" int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out,
     attn_prefill_lds_kernel<M, LDS_QT, LDS_UNITS, true><<<grid, dim3(LDS_UNITS * 2 * WAVE), 0, stream>>>(          \
         (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, qblock_start, qblock_len,       \
         n_qblocks, block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads,         \
-        head_dim, scale, window, hb);                                                                              \
+        head_dim, scale, window, hb, soft_cap);                                                                    \
   else                                                                                                             \
     attn_prefill_lds_kernel<M, LDS_QT, LDS_UNITS, false><<<grid, dim3(LDS_UNITS * 2 * WAVE), 0, stream>>>(         \
       (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, qblock_start, qblock_len,         \
       n_qblocks, block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, \
-      scale, window, hb);                                                                                          \
+      scale, window, hb, soft_cap);                                                                                \
   } while (0)
 #define FMS_PL32(D32)                                                                                              \
   attn_prefill_lds32_kernel<D32, LDS_UNITS><<<grid, dim3(LDS_UNITS * 2 * WAVE), 0, stream>>>(                      \
       (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, qblock_start, qblock_len, n_qblocks, \
-      block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, scale, window, hb)
+      block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, scale, window, hb, soft_cap)
   if (head_dim == 128)  // head sizes with a 32x32x16 kernel of their own
     FMS_PL32(4);
   else if (head_dim == 64)
@@ -1377,7 +1412,7 @@ extern "C" int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, 
                                        const int* block_table, int table_stride, const void* k_cache,
                                        const void* v_cache, int n_tokens, int nheads, int kvheads, int head_dim,
                                        float scale, int window, int max_context, int pages_per_split, int waves,
-                                       int staged, const int* row_order, hipStream_t stream) {
+                                       int staged, const int* row_order, float soft_cap, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   if (check_common("attn_decode_bf16", n_tokens, nheads, kvheads, head_dim, q_stride, out_stride)) return -1;
   FMS_REQUIRE(head_dim % 16 == 0, "attn_decode_bf16: head size %d is no multiple of 16", head_dim);
@@ -1404,7 +1439,7 @@ extern "C" int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, 
   attn_decode_bf16_kernel<M, MAXW, STAGED><<<grid, dim3(waves * WAVE), LDS, stream>>>(                               \
       (const bf16*)q, q_stride, (bf16*)out, out_stride, part_o, part_ml, n_splits, positions, seq_of_token,          \
       block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, scale,       \
-      window, tile_cols, row_order)
+      window, tile_cols, row_order, soft_cap)
   FMS_REQUIRE(staged == 0 || head_dim == 128, "attn_decode_bf16: pages go through LDS for head size 128 only");
   if (staged != 0) {
     // the waves' results meet in the page buffers: 16 KB a wave hold 16 columns of 130 floats

@@ -13,9 +13,10 @@
 //   delta_rule:     the recurrence.  Columns of S never mix (each value channel is a recurrence of its own), so a wave
 //                   owns a few columns of one head of one sequence: 16 lanes share a column, each with a run of its
 //                   rows in registers.  The wave walks over the sequence's tokens; q, k and g of a run of tokens are
-//                   staged in LDS for all its lanes.  With kg = g k and qg = g q, both inner products of a token read
-//                   the state as the token found it,  u = beta (v - S^T kg),  o = S^T qg + (k . q) u,  and are summed
-//                   over the 16 lanes together; then S <- g S + k u^T.
+//                   staged in LDS for all its lanes (the next run's are asked for before this one is worked on).  With
+//                   kg = g k and qg = g q, both inner products of a token read the state as the token found it,
+//                   u = beta (v - S^T kg),  o = S^T qg + (k . q) u,  and are summed over the 16 lanes together, in the
+//                   vector unit; then S <- g S + k u^T.
 //   gated_head_norm: o / rms(o) * weight * act(gate) per head, rounded once to the activation type.
 //
 // The state is kept transposed, [slot][head][value channel][key channel], so that a lane's rows are contiguous.
@@ -33,8 +34,8 @@ __global__ void __launch_bounds__(256)
                          const W* __restrict__ conv_w, int taps, const float* __restrict__ a_log,
                          const float* __restrict__ dt_bias, const float* __restrict__ conv_state,
                          const int* __restrict__ seq_of_token, const int* __restrict__ slot_ids, float* __restrict__ qkv,
-                         float* __restrict__ beta, float* __restrict__ decay, int H, int G, int D, int Dv, int per_channel,
-                         float q_scale) {
+                         float* __restrict__ beta, float* __restrict__ decay, float* __restrict__ kq, int H, int G, int D, int Dv,
+                         int per_channel, float q_scale) {
   extern __shared__ float y[];  // the C convolved channels of this token
   const int t = blockIdx.x;
   const int seq = seq_of_token[t];
@@ -68,6 +69,12 @@ __global__ void __launch_bounds__(256)
     for (int i = lane; i < D; i += WAVE) v[i] *= inv;
   }
   __syncthreads();
+  for (int head = wave; head < G; head += nwaves) {  // k . q of the finished vectors, which the recurrence's read-out needs
+    float s = 0.f;
+    for (int i = lane; i < D; i += WAVE) s = fmaf(y[(size_t)head * D + i], y[(size_t)(G + head) * D + i], s);
+    s = wave_sum(s);
+    if (lane == 0) kq[(size_t)t * G + head] = s;
+  }
   for (int c = threadIdx.x; c < C; c += blockDim.x) qkv[(size_t)t * C + c] = y[c];
   for (int h = threadIdx.x; h < H; h += blockDim.x) beta[(size_t)t * H + h] = sigmoid_f32(proj[(size_t)t * ld + col_b + h]);
   const int per_head = per_channel ? D : 1;
@@ -104,12 +111,15 @@ __global__ void __launch_bounds__(256)
 // the recurrence
 // --------------------------------------------------------------------------
 #define DELTA_PARTS 16                      // lanes that share a column of S
-#define DELTA_COLS (WAVE / DELTA_PARTS)     // columns of S a wave owns
+#define DELTA_WAVES 4                       // waves of a block: they share the staged tokens
+#define DELTA_THREADS (DELTA_WAVES * WAVE)
+#define DELTA_COLS (DELTA_THREADS / DELTA_PARTS)  // columns of S a block owns
 
 struct DeltaArgs {
   const float* qkv;    // [T, C]: q [G*D] | k [G*D] | v [H*Dv]
   const float* beta;   // [T, H]
   const float* decay;  // [T, H] or [T, H*D]
+  const float* kq;     // [T, G]: k . q
   float* state;        // [slots][H][Dv][D]
   float* out;          // [T, H*Dv]
   const int* seq_starts;
@@ -118,24 +128,40 @@ struct DeltaArgs {
   int H, G, D, Dv, per_channel;
 };
 
-// R: rows of S per lane (D <= 16 R).  TC: tokens staged at a time.
-template <int R, int TC>
-__global__ void __launch_bounds__(WAVE) delta_rule_kernel(DeltaArgs a) {
-  constexpr int DP = R * DELTA_PARTS;  // padded key size
+// The sum over the 16 lanes of a row, in all of them, in the vector unit: two swaps inside quads, then the mirror of
+// a half row and of the row (a shuffle through LDS would put four round trips to LDS into every token's chain).
+__device__ __forceinline__ float row16_sum(float v) {
+#define FMS_DPP_ADD(ctrl) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xF, 0xF, true))
+  FMS_DPP_ADD(0xB1);   // quad_perm [1, 0, 3, 2]
+  FMS_DPP_ADD(0x4E);   // quad_perm [2, 3, 0, 1]
+  FMS_DPP_ADD(0x141);  // row_half_mirror
+  FMS_DPP_ADD(0x140);  // row_mirror
+#undef FMS_DPP_ADD
+  return v;
+}
+
+// R: rows of S per lane (D <= 16 R).  TC: tokens staged at a time.  A block's four waves own 16 columns of one head and
+// share the staged tokens (staging costs instructions, and four waves split them).  The next run's q, k and g are
+// asked for from global memory before this run is worked on and wait in registers meanwhile.
+template <int R, int TC, bool PER_CHANNEL>
+__global__ void __launch_bounds__(DELTA_THREADS) delta_rule_kernel(DeltaArgs a) {
+  constexpr int DP = R * DELTA_PARTS;          // padded key size
+  constexpr int NI = TC * DP / DELTA_THREADS;  // staged elements a thread
+  static_assert(TC * DP % DELTA_THREADS == 0 && TC * DELTA_COLS <= DELTA_THREADS, "the staging loops assume this");
   __shared__ __attribute__((aligned(16))) float qg[TC][DP];
   __shared__ __attribute__((aligned(16))) float kg[TC][DP];
   __shared__ __attribute__((aligned(16))) float kk[TC][DP];
   __shared__ __attribute__((aligned(16))) float gg[TC][DP];
   __shared__ float vv[TC][DELTA_COLS];
   __shared__ float bb[TC];
-  __shared__ float kq[TC];
+  __shared__ float kqs[TC];
   __shared__ float oo[TC][DELTA_COLS];
 
   const int b = blockIdx.x, h = blockIdx.y;
   const int t0 = a.seq_starts[b], t1 = a.seq_starts[b + 1];
   if (t0 >= t1 || a.seq_of_token[t0] < 0) return;
   const int slot = a.slot_ids[b];
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x;  // of the block
   const int part = lane % DELTA_PARTS, col = lane / DELTA_PARTS;
   const int j = blockIdx.z * DELTA_COLS + col;  // this lane's column of S
   const int H = a.H, G = a.G, D = a.D, Dv = a.Dv;
@@ -148,67 +174,66 @@ __global__ void __launch_bounds__(WAVE) delta_rule_kernel(DeltaArgs a) {
 #pragma unroll
   for (int r = 0; r < R; ++r) S[r] = (live && part * R + r < D) ? srow[r] : 0.f;
 
+  // what a lane fetches of a run: NI (q, k, g) triples, one value, and beta and k . q of one token
+  float pq[NI], pk[NI], pg[NI], pv = 0.f, pb = 0.f, pkq = 0.f;
+  const int vt = lane / DELTA_COLS, vc = lane % DELTA_COLS;  // the (token, column) whose value and output this lane moves
+  const int vj = blockIdx.z * DELTA_COLS + vc;
+  auto fetch = [&](int tb) {
+#pragma unroll
+    for (int it = 0; it < NI; ++it) {
+      const int idx = it * DELTA_THREADS + lane;
+      const int tt = idx / DP, i = idx % DP;
+      const int t = tb + tt;
+      pq[it] = pk[it] = pg[it] = 0.f;
+      if (t < t1 && i < D) {
+        const float* row = a.qkv + (size_t)t * C;
+        pq[it] = row[kh * D + i];
+        pk[it] = row[G * D + kh * D + i];
+        pg[it] = PER_CHANNEL ? a.decay[((size_t)t * H + h) * D + i] : a.decay[(size_t)t * H + h];
+      }
+    }
+    pv = (vt < TC && tb + vt < t1 && vj < Dv) ? a.qkv[(size_t)(tb + vt) * C + 2 * G * D + h * Dv + vj] : 0.f;
+    if (lane < TC && tb + lane < t1) {
+      pb = a.beta[(size_t)(tb + lane) * H + h];
+      pkq = a.kq[(size_t)(tb + lane) * G + kh];
+    }
+  };
+  fetch(t0);
+
   for (int tb = t0; tb < t1; tb += TC) {
     const int n = t1 - tb < TC ? t1 - tb : TC;
-    __syncthreads();  // the last run's reads are done
-    for (int idx = lane; idx < n * DP; idx += WAVE) {
-      const int tt = idx / DP, i = idx % DP;
-      float q = 0.f, k = 0.f, g = 0.f;
-      if (i < D) {
-        const float* row = a.qkv + (size_t)(tb + tt) * C;
-        q = row[kh * D + i];
-        k = row[G * D + kh * D + i];
-        g = a.per_channel ? a.decay[((size_t)(tb + tt) * H + h) * D + i] : a.decay[(size_t)(tb + tt) * H + h];
-      }
-      qg[tt][i] = q * g;
-      kg[tt][i] = k * g;
-      kk[tt][i] = k;
-      gg[tt][i] = g;
-    }
-    for (int idx = lane; idx < n * DELTA_COLS; idx += WAVE) {
-      const int tt = idx / DELTA_COLS, c = idx % DELTA_COLS;
-      const int jj = blockIdx.z * DELTA_COLS + c;
-      vv[tt][c] = jj < Dv ? a.qkv[(size_t)(tb + tt) * C + 2 * G * D + h * Dv + jj] : 0.f;
-    }
-    if (lane < n) bb[lane] = a.beta[(size_t)(tb + lane) * H + h];
-    // k . q of every staged token: TC tokens x 64 / TC lanes each
-    {
-      constexpr int LPT = WAVE / TC;  // lanes per token
-      const int tt = lane / LPT, sub = lane % LPT;
-      float s = 0.f;
-      if (tt < n) {
-        const float* row = a.qkv + (size_t)(tb + tt) * C;
-        for (int i = sub; i < D; i += LPT) s = fmaf(row[kh * D + i], row[G * D + kh * D + i], s);
-      }
 #pragma unroll
-      for (int off = LPT / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, WAVE);
-      if (sub == 0) kq[tt] = s;
+    for (int it = 0; it < NI; ++it) {
+      const int idx = it * DELTA_THREADS + lane;
+      const int tt = idx / DP, i = idx % DP;
+      qg[tt][i] = pq[it] * pg[it];
+      kg[tt][i] = pk[it] * pg[it];
+      kk[tt][i] = pk[it];
+      gg[tt][i] = pg[it];
     }
-    __syncthreads();
+    if (vt < TC) vv[vt][vc] = pv;
+    if (lane < TC) bb[lane] = pb, kqs[lane] = pkq;
+    block_sync_lds();
+    if (tb + TC < t1) fetch(tb + TC);  // under way while this run is worked on
 
     for (int tt = 0; tt < n; ++tt) {
-      float du = 0.f, dq = 0.f;
+      float du0 = 0.f, du1 = 0.f, dq0 = 0.f, dq1 = 0.f;
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
-        du = fmaf(S[r], kg[tt][part * R + r], du);
-        dq = fmaf(S[r], qg[tt][part * R + r], dq);
+      for (int r = 0; r < R; r += 2) {
+        du0 = fmaf(S[r], kg[tt][part * R + r], du0);
+        dq0 = fmaf(S[r], qg[tt][part * R + r], dq0);
+        du1 = fmaf(S[r + 1], kg[tt][part * R + r + 1], du1);
+        dq1 = fmaf(S[r + 1], qg[tt][part * R + r + 1], dq1);
       }
-#pragma unroll
-      for (int off = DELTA_PARTS / 2; off > 0; off >>= 1) {
-        du += __shfl_xor(du, off, WAVE);
-        dq += __shfl_xor(dq, off, WAVE);
-      }
+      const float du = row16_sum(du0 + du1), dq = row16_sum(dq0 + dq1);
       const float u = bb[tt] * (vv[tt][col] - du);
 #pragma unroll
       for (int r = 0; r < R; ++r) S[r] = fmaf(kk[tt][part * R + r], u, gg[tt][part * R + r] * S[r]);
-      if (part == 0) oo[tt][col] = fmaf(kq[tt], u, dq);
+      if (part == 0) oo[tt][col] = fmaf(kqs[tt], u, dq);
     }
-    __syncthreads();
-    for (int idx = lane; idx < n * DELTA_COLS; idx += WAVE) {
-      const int tt = idx / DELTA_COLS, c = idx % DELTA_COLS;
-      const int jj = blockIdx.z * DELTA_COLS + c;
-      if (jj < Dv) a.out[(size_t)(tb + tt) * H * Dv + h * Dv + jj] = oo[tt][c];
-    }
+    block_sync_lds();
+    if (vt < n && vj < Dv) a.out[(size_t)(tb + vt) * H * Dv + h * Dv + vj] = oo[vt][vc];
+    block_sync_lds();  // the run's reads are done before the next one is written
   }
   if (live) {
 #pragma unroll
@@ -243,8 +268,8 @@ __global__ void __launch_bounds__(256)
 extern "C" int fmsamd_delta_prepare(const float* proj, long ld, int col_b, const float* a, long lda, int col_a, const void* conv_w,
                                     int conv_dtype, int taps, const float* a_log, const float* dt_bias, float* conv_state,
                                     const int* seq_of_token, const int* slot_ids, float* qkv, float* beta, float* decay,
-                                    int n_tokens, int heads, int kv_heads, int dim, int vdim, int per_channel, float q_scale,
-                                    hipStream_t stream) {
+                                    float* kq, int n_tokens, int heads, int kv_heads, int dim, int vdim, int per_channel,
+                                    float q_scale, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   FMS_REQUIRE(n_tokens > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0,
               "delta_prepare: bad sizes heads=%d kv_heads=%d dim=%d vdim=%d", heads, kv_heads, dim, vdim);
@@ -257,7 +282,7 @@ extern "C" int fmsamd_delta_prepare(const float* proj, long ld, int col_b, const
 #define FMS_PREP(W)                                                                                                   \
   delta_prepare_kernel<W><<<n_tokens, 256, lds, stream>>>(proj, ld, col_b, a, lda, col_a, (const W*)conv_w, taps, a_log, \
                                                           dt_bias, conv_state, seq_of_token, slot_ids, qkv, beta, decay, \
-                                                          heads, kv_heads, dim, vdim, per_channel, q_scale)
+                                                          kq, heads, kv_heads, dim, vdim, per_channel, q_scale)
   if (conv_dtype == FMS_F32) FMS_PREP(float);
   else if (conv_dtype == FMS_BF16) FMS_PREP(bf16);
   else FMS_REQUIRE(false, "delta_prepare: unknown dtype %d", conv_dtype);
@@ -270,20 +295,26 @@ extern "C" int fmsamd_delta_prepare(const float* proj, long ld, int col_b, const
   return 0;
 }
 
-extern "C" int fmsamd_delta_rule(const float* qkv, const float* beta, const float* decay, float* state, float* out,
-                                 const int* seq_starts, const int* seq_of_token, const int* slot_ids, int n_seqs, int heads,
+extern "C" int fmsamd_delta_rule(const float* qkv, const float* beta, const float* decay, const float* kq, float* state,
+                                 float* out, const int* seq_starts, const int* seq_of_token, const int* slot_ids, int n_seqs, int heads,
                                  int kv_heads, int dim, int vdim, int per_channel, hipStream_t stream) {
   if (n_seqs == 0) return 0;
   FMS_REQUIRE(n_seqs > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0,
               "delta_rule: bad sizes heads=%d kv_heads=%d dim=%d vdim=%d", heads, kv_heads, dim, vdim);
   FMS_REQUIRE(dim <= 16 * DELTA_PARTS, "delta_rule: %d key channels (at most %d)", dim, 16 * DELTA_PARTS);
   FMS_REQUIRE(heads <= 65535 && ceil_div(vdim, DELTA_COLS) <= 65535, "delta_rule: too many heads or value channels for one launch");
-  DeltaArgs a{qkv, beta, decay, state, out, seq_starts, seq_of_token, slot_ids, heads, kv_heads, dim, vdim, per_channel};
+  DeltaArgs a{qkv, beta, decay, kq, state, out, seq_starts, seq_of_token, slot_ids, heads, kv_heads, dim, vdim, per_channel};
   const dim3 grid(n_seqs, heads, ceil_div(vdim, DELTA_COLS));
-  if (dim <= 2 * DELTA_PARTS) delta_rule_kernel<2, 16><<<grid, WAVE, 0, stream>>>(a);
-  else if (dim <= 4 * DELTA_PARTS) delta_rule_kernel<4, 16><<<grid, WAVE, 0, stream>>>(a);
-  else if (dim <= 8 * DELTA_PARTS) delta_rule_kernel<8, 16><<<grid, WAVE, 0, stream>>>(a);
-  else delta_rule_kernel<16, 8><<<grid, WAVE, 0, stream>>>(a);
+#define FMS_DR(R, TC)                                                                       \
+  do {                                                                                      \
+    if (per_channel) delta_rule_kernel<R, TC, true><<<grid, DELTA_THREADS, 0, stream>>>(a);   \
+    else delta_rule_kernel<R, TC, false><<<grid, DELTA_THREADS, 0, stream>>>(a);  \
+  } while (0)
+  if (dim <= 2 * DELTA_PARTS) FMS_DR(2, 16);
+  else if (dim <= 4 * DELTA_PARTS) FMS_DR(4, 16);
+  else if (dim <= 8 * DELTA_PARTS) FMS_DR(8, 16);
+  else FMS_DR(16, 8);
+#undef FMS_DR
   FMS_LAUNCH_CHECK("delta_rule");
   return 0;
 }

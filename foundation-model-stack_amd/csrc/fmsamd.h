@@ -70,6 +70,7 @@ int fmsamd_attn_generic(const void* q, long q_stride, void* out, long out_stride
                         const void* v_cache, int n_tokens, int nheads, int kvheads, int head_dim, float scale,
                         int window, const float* slopes, float soft_cap, int value_dim, hipStream_t stream);
 
+// soft_cap (0: none) of the two bfloat16 kernels: scores become soft_cap * tanh(score / soft_cap).
 // bfloat16 prefill: the step is cut into query blocks of at most fmsamd_attn_prefill_qblock(...) consecutive
 // tokens of one sequence; the same number goes into the call as qblock_tokens
 int fmsamd_attn_prefill_qblock(int nheads, int kvheads, int head_dim, int n_tokens);
@@ -77,7 +78,7 @@ int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out, long out_s
                              const int* seq_of_token, const int* qblock_start, const int* qblock_len, int n_qblocks,
                              int qblock_tokens, const int* block_table, int table_stride, const void* k_cache, const void* v_cache,
                              int n_tokens, int nheads, int kvheads, int head_dim, float scale, int window,
-                             hipStream_t stream);
+                             float soft_cap, hipStream_t stream);
 
 // bfloat16 decode: one token per sequence.  The context bound max_context is cut into splits of
 // `pages_per_split` pages, and every sequence deals its own pages out evenly over that many blocks of `waves`
@@ -91,7 +92,7 @@ int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, long out_st
                             const int* block_table, int table_stride, const void* k_cache, const void* v_cache,
                             int n_tokens, int nheads, int kvheads, int head_dim, float scale, int window,
                             int max_context, int pages_per_split, int waves, int staged, const int* row_order,
-                            hipStream_t stream);
+                            float soft_cap, hipStream_t stream);
 
 // c[M, N] = a[M, K] w[N, K]^T (+ bias[N])
 int fmsamd_gemm_f32(const float* a, long lda, const float* w, const float* bias, float* c, long ldc, int M, int N,
@@ -257,14 +258,15 @@ int fmsamd_scale_f32(float* x, long n, float s, hipStream_t stream);
 // convolution and whose columns col_b .. col_b + heads are the logits of beta; a: rows with the decay's input at col_a
 // (heads columns, or heads*dim if per_channel); conv_w [C, taps]; conv_state [slots][taps-1][C] is read, then updated.
 // Writes qkv [T, C] (convolved, silu, q and k unit vectors per head, q times q_scale), beta [T, heads] and
-// decay [T, heads (*dim)] = exp(-exp(a_log) softplus(a + dt_bias)).
+// decay [T, heads (*dim)] = exp(-exp(a_log) softplus(a + dt_bias)), and kq [T, kv_heads] = k . q of the finished vectors.
 int fmsamd_delta_prepare(const float* proj, long ld, int col_b, const float* a, long lda, int col_a, const void* conv_w,
                          int conv_dtype, int taps, const float* a_log, const float* dt_bias, float* conv_state,
-                         const int* seq_of_token, const int* slot_ids, float* qkv, float* beta, float* decay, int n_tokens,
-                         int heads, int kv_heads, int dim, int vdim, int per_channel, float q_scale, hipStream_t stream);
+                         const int* seq_of_token, const int* slot_ids, float* qkv, float* beta, float* decay, float* kq,
+                         int n_tokens, int heads, int kv_heads, int dim, int vdim, int per_channel, float q_scale,
+                         hipStream_t stream);
 // The recurrence over every sequence's tokens of the step (seq_starts [n_seqs + 1]); state [slots][heads][vdim][dim]
 // is read and written; out [T, heads*vdim].
-int fmsamd_delta_rule(const float* qkv, const float* beta, const float* decay, float* state, float* out,
+int fmsamd_delta_rule(const float* qkv, const float* beta, const float* decay, const float* kq, float* state, float* out,
                       const int* seq_starts, const int* seq_of_token, const int* slot_ids, int n_seqs, int heads,
                       int kv_heads, int dim, int vdim, int per_channel, hipStream_t stream);
 // out[t, h, :] = o[t, h, :] / rms * weight * act(gate[t, h, :]) * out_scale

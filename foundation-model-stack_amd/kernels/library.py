@@ -34,8 +34,8 @@ _SIGNATURES = {
     "fmsamd_rope_table": [P, P, P, I, I, P],
     "fmsamd_rope_kv_write": [P, I, L, P, P, P, I, P, P, I, I, P, P, I, I, I, I, I, P],
     "fmsamd_attn_generic": [P, L, P, L, I, P, P, P, I, P, P, I, I, I, I, F, I, P, F, I, P],
-    "fmsamd_attn_prefill_bf16": [P, L, P, L, P, P, P, P, I, I, P, I, P, P, I, I, I, I, F, I, P],
-    "fmsamd_attn_decode_bf16": [P, L, P, L, P, L, P, P, P, I, P, P, I, I, I, I, F, I, I, I, I, I, P, P],
+    "fmsamd_attn_prefill_bf16": [P, L, P, L, P, P, P, P, I, I, P, I, P, P, I, I, I, I, F, I, F, P],
+    "fmsamd_attn_decode_bf16": [P, L, P, L, P, L, P, P, P, I, P, P, I, I, I, I, F, I, I, I, I, I, P, F, P],
     "fmsamd_qkv_rope_skinny_bf16": [P, L, P, P, I, P, L, I, I, P, P, P, I, P, P, I, I, P, P, I, I, I, P, P, L, P],
     "fmsamd_gemm_f32": [P, L, P, P, P, L, I, I, I, P],
     "fmsamd_gemm_bf16": [P, L, P, P, I, P, I, L, I, I, I, P],
@@ -62,8 +62,8 @@ _SIGNATURES = {
     "fmsamd_qk_projection_norm": [P, L, I, I, I, P, P, I, F, P, I, L, P, I, P],
     "fmsamd_gate_mul": [P, L, P, L, I, F, P, L, I, I, I, P],
     "fmsamd_scale_f32": [P, L, F, P],
-    "fmsamd_delta_prepare": [P, L, I, P, L, I, P, I, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, P],
-    "fmsamd_delta_rule": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
+    "fmsamd_delta_prepare": [P, L, I, P, L, I, P, I, I, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, P],
+    "fmsamd_delta_rule": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P],
     "fmsamd_gated_head_norm": [P, P, L, P, I, F, I, F, P, I, L, P, I, I, I, P],
     "fmsamd_moe_combine": [P, P, I, P, P, L, P, I, I, I, P],
     "fmsamd_probe_read": [P, L, I, I, P, P],

@@ -350,7 +350,8 @@ def attention(
 
     Further terms of the scores (a position encoding that acts on the scores, a capped attention): score_slopes,
     float32 [nheads], adds slope[head] * (key position - query position); soft_cap c > 0 turns a score s into
-    c * tanh(s / c) first.  With either, both types run the generic kernel (the MFMA kernels have no such term).
+    c * tanh(s / c) first.  With slopes both types run the generic kernel (the MFMA kernels have no such term); the
+    cap they have.
 
     q is a [T, >= nheads*head_dim] view (the query columns of the qkv rows).  float32 runs the
     generic kernel; bfloat16 runs the MFMA kernels (prefill needs the query blocks, decode the
@@ -372,7 +373,7 @@ def attention(
             raise ValueError(f"score_slopes must be a contiguous float32 [{nheads}] tensor")
     if not (soft_cap >= 0.0 and math.isfinite(soft_cap)):
         raise ValueError(f"soft_cap {soft_cap} must be zero (none) or positive")
-    if q.dtype == torch.float32 or force_generic or head_dim % 16 or score_slopes is not None or soft_cap > 0.0 or value_dim:
+    if q.dtype == torch.float32 or force_generic or head_dim % 16 or score_slopes is not None or value_dim:
         for t0 in range(0, T, 65535):
             n = min(65535, T - t0)
             check(lib.fmsamd_attn_generic(q[t0:].data_ptr(), q.stride(0), out[t0:].data_ptr(), out.stride(0), _code(q.dtype),
@@ -401,7 +402,8 @@ def attention(
                                           positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
                                           block_table.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), T, nheads, kvheads,
                                           head_dim, float(scale), int(window), int(max_context), int(pages_per_block), int(waves),
-                                          int(bool(staged)) if staged is not None else int(head_dim == 128), _ptr(row_order), _stream()))
+                                          int(bool(staged)) if staged is not None else int(head_dim == 128), _ptr(row_order),
+                                          float(soft_cap), _stream()))
         return out
     if qblock_start is None or qblock_len is None:
         raise ValueError("bfloat16 prefill attention needs the query blocks of the batch")
@@ -410,7 +412,7 @@ def attention(
     check(lib.fmsamd_attn_prefill_bf16(q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), positions.data_ptr(),
                                        seq_of_token.data_ptr(), qblock_start.data_ptr(), qblock_len.data_ptr(),
                                        qblock_start.numel(), int(qblock_tokens), block_table.data_ptr(), block_table.stride(0),
-                                       k_cache.data_ptr(), v_cache.data_ptr(), *common_tail))
+                                       k_cache.data_ptr(), v_cache.data_ptr(), *common_tail[:-1], float(soft_cap), common_tail[-1]))
     return out
 
 
@@ -972,7 +974,7 @@ def delta_prepare(proj: torch.Tensor, col_b: int, a: torch.Tensor, col_a: int, c
                   dt_bias: torch.Tensor, conv_state: torch.Tensor, seq_of_token: torch.Tensor, slot_ids: torch.Tensor, heads: int,
                   kv_heads: int, dim: int, vdim: int, per_channel: bool, q_scale: float):
     """What the recurrence of a step reads, from the float32 projections of its tokens: (qkv [T, C], beta [T, heads],
-    decay [T, heads] or [T, heads*dim]), all float32.  The first C = 2*kv_heads*dim + heads*vdim columns of `proj` pass the
+    decay [T, heads] or [T, heads*dim], kq [T, kv_heads] = k . q), all float32.  The first C = 2*kv_heads*dim + heads*vdim columns of `proj` pass the
     short causal convolution (conv_w [C, taps]; the inputs before the step come from conv_state [slots, taps-1, C], which
     is then moved on), silu, and q and k become unit vectors per head (q times q_scale); beta = sigmoid(proj[:, col_b:]);
     decay = exp(-exp(a_log) * softplus(a[:, col_a:] + dt_bias))."""
@@ -1002,26 +1004,27 @@ def delta_prepare(proj: torch.Tensor, col_b: int, a: torch.Tensor, col_a: int, c
     qkv = torch.empty(T, C, dtype=torch.float32, device=proj.device)
     beta = torch.empty(T, heads, dtype=torch.float32, device=proj.device)
     decay = torch.empty(T, heads * per, dtype=torch.float32, device=proj.device)
+    kq = torch.empty(T, kv_heads, dtype=torch.float32, device=proj.device)
     check(load().fmsamd_delta_prepare(proj.data_ptr(), proj.stride(0), col_b, a.data_ptr(), a.stride(0), col_a, conv_w.data_ptr(),
                                       _code(conv_w.dtype), taps, a_log.data_ptr(), dt_bias.data_ptr(), conv_state.data_ptr(),
                                       seq_of_token.data_ptr(), slot_ids.data_ptr(), qkv.data_ptr(), beta.data_ptr(), decay.data_ptr(),
-                                      T, heads, kv_heads, dim, vdim, int(bool(per_channel)), float(q_scale), _stream()))
-    return qkv, beta, decay
+                                      kq.data_ptr(), T, heads, kv_heads, dim, vdim, int(bool(per_channel)), float(q_scale), _stream()))
+    return qkv, beta, decay, kq
 
 
-def delta_rule(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, state: torch.Tensor, seq_starts: torch.Tensor,
+def delta_rule(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, kq: torch.Tensor, state: torch.Tensor, seq_starts: torch.Tensor,
                seq_of_token: torch.Tensor, slot_ids: torch.Tensor, n_seqs: int, heads: int, kv_heads: int, dim: int, vdim: int,
                per_channel: bool) -> torch.Tensor:
     """The recurrence S = g S; u = beta (v - S^T k); S += k u^T; o = S^T q over the tokens of every sequence of the
-    step, from and into state [slots, heads, vdim, dim] (float32, S transposed) -> o float32 [T, heads*vdim].
+    step (kq [T, kv_heads] holds k . q of every token, as delta_prepare leaves it), from and into state [slots, heads, vdim, dim] (float32, S transposed) -> o float32 [T, heads*vdim].
     Sequence b of the step owns the token rows seq_starts[b] .. seq_starts[b + 1] and the state of slot_ids[b]."""
-    _need_cuda(qkv, beta, decay, state, seq_starts, seq_of_token, slot_ids)
+    _need_cuda(qkv, beta, decay, kq, state, seq_starts, seq_of_token, slot_ids)
     for name, t in (("seq_starts", seq_starts), ("seq_of_token", seq_of_token), ("slot_ids", slot_ids)):
         _need_i32(name, t)
     T = qkv.shape[0]
     C = 2 * kv_heads * dim + heads * vdim
     per = dim if per_channel else 1
-    for name, t, cols in (("qkv", qkv, C), ("beta", beta, heads), ("decay", decay, heads * per)):
+    for name, t, cols in (("qkv", qkv, C), ("beta", beta, heads), ("decay", decay, heads * per), ("kq", kq, kv_heads)):
         if t.dtype != torch.float32 or tuple(t.shape) != (T, cols) or not t.is_contiguous():
             raise ValueError(f"{name} is contiguous float32 [{T}, {cols}]")
     if state.dtype != torch.float32 or state.dim() != 4 or tuple(state.shape[1:]) != (heads, vdim, dim) or not state.is_contiguous():
@@ -1031,7 +1034,7 @@ def delta_rule(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, state
     if seq_starts.numel() < n_seqs + 1 or slot_ids.numel() < n_seqs or seq_of_token.numel() < T:
         raise ValueError("the step's index arrays are shorter than its sequences or tokens")
     out = torch.empty(T, heads * vdim, dtype=torch.float32, device=qkv.device)
-    check(load().fmsamd_delta_rule(qkv.data_ptr(), beta.data_ptr(), decay.data_ptr(), state.data_ptr(), out.data_ptr(),
+    check(load().fmsamd_delta_rule(qkv.data_ptr(), beta.data_ptr(), decay.data_ptr(), kq.data_ptr(), state.data_ptr(), out.data_ptr(),
                                    seq_starts.data_ptr(), seq_of_token.data_ptr(), slot_ids.data_ptr(), n_seqs, heads, kv_heads, dim,
                                    vdim, int(bool(per_channel)), _stream()))
     return out

@@ -116,8 +116,7 @@ class MultiHeadAttention(Mixer):
         return self.position_encoder.score_slopes(self.nheads) if self.position_encoder is not None else None
 
     def prefill_qblock(self, n_tokens: int, dtype) -> int:
-        if (dtype != torch.bfloat16 or self.head_dim % 16 or self.soft_cap > 0 or self._score_slopes() is not None
-                or self.value_dim != self.head_dim):
+        if dtype != torch.bfloat16 or self.head_dim % 16 or self._score_slopes() is not None or self.value_dim != self.head_dim:
             return 0  # the generic kernel takes tokens one by one
         return ops.prefill_qblock(self.nheads, self.kvheads, self.head_dim, n_tokens)
 

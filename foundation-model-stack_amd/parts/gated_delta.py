@@ -112,9 +112,9 @@ class GatedDeltaRule(Mixer):
             gate = self.gate_up.forward(low, out_dtype=torch.float32)
         else:
             gate = proj[:, self.col_g : self.col_g + H * V]
-        qkv, beta, decay = ops.delta_prepare(proj, self.col_b, a, col_a, self.w["conv.weight"], self._a_log, self._dt_bias,
+        qkv, beta, decay, kq = ops.delta_prepare(proj, self.col_b, a, col_a, self.w["conv.weight"], self._a_log, self._dt_bias,
                                              state["conv"], batch.seq_of_token, batch.slot_ids, H, G, D, V, self.per_channel, D ** -0.5)
-        o = ops.delta_rule(qkv, beta, decay, state["S"], batch.seq_starts, batch.seq_of_token, batch.slot_ids, batch.n_seqs, H, G, D, V,
+        o = ops.delta_rule(qkv, beta, decay, kq, state["S"], batch.seq_starts, batch.seq_of_token, batch.slot_ids, batch.n_seqs, H, G, D, V,
                            self.per_channel)
         normed = ops.gated_head_norm(o, gate, self.w["norm.weight"], self.eps, self.gate_activation, H, V, x.dtype, batch.seq_of_token,
                                      scale=out_scale, out=out)

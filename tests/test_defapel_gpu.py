@@ -76,6 +76,11 @@ CONFIGS = {
         parallel(attention(8, 2, 64, 64, 128, 32, base=500000.0, scaling=(8.0, 1.0, 4.0, 64)), delta(4, 2, 128, 64, 4), 0.9, 0.8, moe(8, 2, 128)),
         channel(delta(4, 4, 64, 128, 4, ranks=(16, 16)), moe(8, 2, 128)),
     ]),
+    # the other head sizes with matrix-instruction attention kernels of their own: 128 and 32; 256 key channels a head
+    "D": dict(vocab=400, width=256, norm={"eps": 1e-6}, logit_scale=2.5, max_positions=2048, layers=[
+        parallel(attention(4, 2, 128, 128, 100, 64, base=50000.0, softcap=25.0), delta(2, 1, 256, 32, 4), 1.0, 0.6, moe(4, 1, 64)),
+        parallel(attention(8, 8, 32, 32, 64, 32, softcap=10.0), delta(8, 8, 32, 32, 4), 0.5, 1.0, None),
+    ]),
 }
 
 
@@ -271,9 +276,9 @@ def test_delta_rule_whole_in_portions_and_in_a_batch(lib, sizes):
         slot_ids = torch.tensor(slots, dtype=torch.int32, device=DEV)
         pr = torch.cat([p for p, _ in pieces]).to(DEV)
         aa = torch.cat([x for _, x in pieces]).to(DEV)
-        qkv, beta, decay = ops.delta_prepare(pr, C, aa, 1, conv_w.to(DEV), a_log.to(DEV), dt_bias.to(DEV), conv_state, seq, slot_ids,
-                                             H, G, D, V, per_channel, D ** -0.5)
-        out = ops.delta_rule(qkv, beta, decay, S, starts, seq, slot_ids, len(pieces), H, G, D, V, per_channel)
+        qkv, beta, decay, kq = ops.delta_prepare(pr, C, aa, 1, conv_w.to(DEV), a_log.to(DEV), dt_bias.to(DEV), conv_state, seq, slot_ids,
+                                                 H, G, D, V, per_channel, D ** -0.5)
+        out = ops.delta_rule(qkv, beta, decay, kq, S, starts, seq, slot_ids, len(pieces), H, G, D, V, per_channel)
         return torch.split(out.cpu(), lens)
 
     tol = dict(atol=5e-5, rtol=1e-4)
@@ -297,9 +302,9 @@ def test_delta_rule_whole_in_portions_and_in_a_batch(lib, sizes):
     # a padding row (sequence -1) between live ones changes nothing and writes no state
     before = S.clone()
     seq = torch.tensor([-1], dtype=torch.int32, device=DEV)
-    qkv, beta, decay = ops.delta_prepare(proj[:1].to(DEV), C, a[:1].to(DEV), 1, conv_w.to(DEV), a_log.to(DEV), dt_bias.to(DEV), conv_state,
-                                         seq, torch.tensor([2], dtype=torch.int32, device=DEV), H, G, D, V, per_channel, 1.0)
-    ops.delta_rule(qkv, beta, decay, S, torch.tensor([0, 1], dtype=torch.int32, device=DEV), seq,
+    qkv, beta, decay, kq = ops.delta_prepare(proj[:1].to(DEV), C, a[:1].to(DEV), 1, conv_w.to(DEV), a_log.to(DEV), dt_bias.to(DEV), conv_state,
+                                             seq, torch.tensor([2], dtype=torch.int32, device=DEV), H, G, D, V, per_channel, 1.0)
+    ops.delta_rule(qkv, beta, decay, kq, S, torch.tensor([0, 1], dtype=torch.int32, device=DEV), seq,
                    torch.tensor([2], dtype=torch.int32, device=DEV), 1, H, G, D, V, per_channel)
     assert bool((S == before).all())
 
@@ -323,15 +328,16 @@ def test_a_lost_state_shows(lib):
     starts = torch.tensor([0, T], dtype=torch.int32, device=DEV)
     slot = torch.zeros(1, dtype=torch.int32, device=DEV)
     S = torch.zeros(1, H, V, D, device=DEV)
-    got = ops.delta_rule(qkv.to(DEV), beta.to(DEV), decay.to(DEV), S, starts, seq, slot, 1, H, G, D, V, False).cpu()
+    kq = (qkv[:, :D] * keys).sum(-1, keepdim=True)
+    got = ops.delta_rule(qkv.to(DEV), beta.to(DEV), decay.to(DEV), kq.to(DEV), S, starts, seq, slot, 1, H, G, D, V, False).cpu()
     torch.testing.assert_close(got, want.view(T, V), atol=1e-4, rtol=1e-4)
     # the first token's value still holds a good part of the last read-out
     assert float((want[-1, 0] - 0).norm()) > 0.1
     S.zero_()
-    first = ops.delta_rule(qkv[:300].to(DEV), beta[:300].to(DEV), decay[:300].to(DEV), S, torch.tensor([0, 300], dtype=torch.int32, device=DEV),
+    first = ops.delta_rule(qkv[:300].to(DEV), beta[:300].to(DEV), decay[:300].to(DEV), kq[:300].to(DEV), S, torch.tensor([0, 300], dtype=torch.int32, device=DEV),
                            seq[:300], slot, 1, H, G, D, V, False)
     S.zero_()  # the state is lost between two steps
-    rest = ops.delta_rule(qkv[300:].to(DEV), beta[300:].to(DEV), decay[300:].to(DEV), S, torch.tensor([0, 100], dtype=torch.int32, device=DEV),
+    rest = ops.delta_rule(qkv[300:].to(DEV), beta[300:].to(DEV), decay[300:].to(DEV), kq[300:].to(DEV), S, torch.tensor([0, 100], dtype=torch.int32, device=DEV),
                           seq[:100], slot, 1, H, G, D, V, False).cpu()
     assert float((rest - want.view(T, V)[300:]).abs().max()) > 0.05 and first.shape[0] == 300
 
