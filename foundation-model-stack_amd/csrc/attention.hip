@@ -96,19 +96,19 @@ __global__ void __launch_bounds__(GEN_THREADS)
 
 // What turns a raw score q . k into the exponent of its probability: scale2 = softmax scale * log2(e), and, for capped
 // scores (score = cap * tanh(scale * q . k / cap)), the two factors of a transformation of the raw score that leaves the
-// rest of the softmax as it is: raw' = cap_out * tanh(raw * cap_in), cap_in = scale / cap, cap_out = cap / scale.
+// rest of the softmax as it is: raw' = tanh(raw * cap_in) / cap_in, cap_in = scale / cap.
 // cap_in 0: no cap (a uniform branch that costs nothing).
 struct Scale2 {
-  float v, cap_in, cap_out;
+  float v, cap_in;
   __device__ __forceinline__ operator float() const { return v; }
 };
 __device__ __forceinline__ Scale2 make_scale2(float scale, float soft_cap) {
-  return Scale2{scale * LOG2E, soft_cap > 0.f ? scale / soft_cap : 0.f, soft_cap > 0.f ? soft_cap / scale : 0.f};
+  return Scale2{scale * LOG2E, soft_cap > 0.f ? scale / soft_cap : 0.f};
 }
 // tanh from the hardware's exponential and reciprocal: 1 - 2 / (1 + e^(2x)); exact at both ends (e^(2x) = inf or 0)
 __device__ __forceinline__ float capped(float raw, Scale2 s) {
   const float e = __builtin_amdgcn_exp2f(raw * (s.cap_in * 2.f * LOG2E));
-  return s.cap_out * (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + e));
+  return __builtin_amdgcn_rcpf(s.cap_in) * (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + e));
 }
 // the maximum that a partial result of the decode kernel carries when it holds no key at all
 #define DECODE_EMPTY -1e30f
@@ -542,7 +542,10 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
       const int key0 = pi * PAGE_TOKENS + khalf * 32;
       if (has_work && pi <= page_last && !(key0 > wave_hi || key0 + 31 < wave_lo))  // uniform over the wave
         half_step<MAXDT, QT>(st, qreg, qpos, qlo, key0, ks + cur * PAGE_ELEMS + khalf * 32 * KS, KS,
-                             vs + cur * PAGE_ELEMS + khalf * 32, VS, head_dim, make_scale2(scale, soft_cap),
+                             vs + cur * PAGE_ELEMS + khalf * 32, VS, head_dim,
+                             // the kernel for head sizes between 64 and 128 has no register left for the cap (the host sends
+                             // capped scores of such heads to the generic kernel)
+                             make_scale2(scale, (MAXDT == 8 && !EXACT) ? 0.f : soft_cap),
                              key0 + 31 <= full_hi && key0 >= full_lo);
       block_sync_lds();  // the page just multiplied is overwritten after the next one
     }
@@ -1364,6 +1367,8 @@ extern "C" int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out,
     FMS_LAUNCH_CHECK("attn_prefill_bf16");
     return 0;
   }
+  FMS_REQUIRE(!(soft_cap > 0.f && head_dim > 64 && head_dim < 128),
+              "attn_prefill_bf16: capped scores of head size %d go through attn_generic", head_dim);
   int hb, qt_unused, qblock_expected;
   prefill_shape(nheads, kvheads, head_dim, n_tokens, &hb, &qt_unused, &qblock_expected);
   FMS_REQUIRE(qblock_tokens == qblock_expected, "attn_prefill_bf16: query blocks of %d tokens, %d expected",

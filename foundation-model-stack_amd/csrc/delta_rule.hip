@@ -49,14 +49,31 @@ __global__ void __launch_bounds__(256)
     else break;
   }
   const float* state = conv_state + (size_t)slot * (taps - 1) * C;
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
-    float acc = 0.f;
-    for (int j = 0; j < taps; ++j) {
-      const int d = taps - 1 - j;  // how far back this tap reaches
-      const float x = d <= have ? proj[(size_t)(t - d) * ld + c] : state[(size_t)(taps - 1 + have - d) * C + c];
-      acc = fmaf(to_f32(conv_w[(size_t)c * taps + j]), x, acc);
+  // two channels a thread and pass, all their taps asked for before any is used: a decode step has a block per token
+  // and nothing else to hide a load's latency behind
+  for (int c0 = threadIdx.x; c0 < C; c0 += 2 * blockDim.x) {
+    float x[2][DELTA_MAX_TAPS], w[2][DELTA_MAX_TAPS];
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int c = c0 + e * blockDim.x;
+#pragma unroll
+      for (int j = 0; j < DELTA_MAX_TAPS; ++j) {
+        const int d = taps - 1 - j;  // how far back this tap reaches
+        x[e][j] = w[e][j] = 0.f;
+        if (j < taps && c < C) {
+          x[e][j] = d <= have ? proj[(size_t)(t - d) * ld + c] : state[(size_t)(taps - 1 + have - d) * C + c];
+          w[e][j] = to_f32(conv_w[(size_t)c * taps + j]);
+        }
+      }
     }
-    y[c] = acc / (1.f + expf(-acc));
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int c = c0 + e * blockDim.x;
+      float acc = 0.f;
+#pragma unroll
+      for (int j = 0; j < DELTA_MAX_TAPS; ++j) acc = fmaf(w[e][j], x[e][j], acc);
+      if (c < C) y[c] = acc / (1.f + expf(-acc));
+    }
   }
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
@@ -85,7 +102,7 @@ __global__ void __launch_bounds__(256)
 }
 
 // Runs after delta_prepare of the same step (which reads the old state).  The block of a sequence's last token of the
-// step writes; new entry s reads either a row of the step or an old entry above s, so ascending order is safe in place.
+// step writes; new entry s is either a row of the step or an old entry above s.
 __global__ void __launch_bounds__(256)
     conv_state_kernel(const float* __restrict__ proj, long ld, int taps, float* __restrict__ conv_state,
                       const int* __restrict__ seq_of_token, const int* __restrict__ slot_ids, int n_tokens, int C) {
@@ -100,10 +117,16 @@ __global__ void __launch_bounds__(256)
   }
   float* state = conv_state + (size_t)slot_ids[seq] * (taps - 1) * C;
   for (int c = threadIdx.x; c < C; c += blockDim.x) {
-    for (int s = 0; s < taps - 1; ++s) {
+    float fresh[DELTA_MAX_TAPS - 1];  // all of a channel's new entries are read before any is written
+#pragma unroll
+    for (int s = 0; s < DELTA_MAX_TAPS - 1; ++s) {
       const int d = taps - 2 - s;  // new entry s is the input d tokens before the last one
-      state[(size_t)s * C + c] = d <= have ? proj[(size_t)(t - d) * ld + c] : state[(size_t)(taps - 1 + have - d) * C + c];
+      fresh[s] = 0.f;
+      if (s < taps - 1) fresh[s] = d <= have ? proj[(size_t)(t - d) * ld + c] : state[(size_t)(taps - 1 + have - d) * C + c];
     }
+#pragma unroll
+    for (int s = 0; s < DELTA_MAX_TAPS - 1; ++s)
+      if (s < taps - 1) state[(size_t)s * C + c] = fresh[s];
   }
 }
 
@@ -216,20 +239,46 @@ __global__ void __launch_bounds__(DELTA_THREADS) delta_rule_kernel(DeltaArgs a) 
     block_sync_lds();
     if (tb + TC < t1) fetch(tb + TC);  // under way while this run is worked on
 
-    for (int tt = 0; tt < n; ++tt) {
+    // a token's operands are read from LDS into registers while the token before it is worked on (two sets, in turn)
+    struct Operands {
+      float kg[R], qg[R], kk[R], gg[R], beta, v, kq;
+    };
+    auto load = [&](Operands& x, int tt) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        x.kg[r] = kg[tt][part * R + r];
+        x.qg[r] = qg[tt][part * R + r];
+        x.kk[r] = kk[tt][part * R + r];
+        x.gg[r] = gg[tt][part * R + r];
+      }
+      x.beta = bb[tt];
+      x.v = vv[tt][col];
+      x.kq = kqs[tt];
+    };
+    auto work = [&](const Operands& x, int tt) {
       float du0 = 0.f, du1 = 0.f, dq0 = 0.f, dq1 = 0.f;
 #pragma unroll
       for (int r = 0; r < R; r += 2) {
-        du0 = fmaf(S[r], kg[tt][part * R + r], du0);
-        dq0 = fmaf(S[r], qg[tt][part * R + r], dq0);
-        du1 = fmaf(S[r + 1], kg[tt][part * R + r + 1], du1);
-        dq1 = fmaf(S[r + 1], qg[tt][part * R + r + 1], dq1);
+        du0 = fmaf(S[r], x.kg[r], du0);
+        dq0 = fmaf(S[r], x.qg[r], dq0);
+        du1 = fmaf(S[r + 1], x.kg[r + 1], du1);
+        dq1 = fmaf(S[r + 1], x.qg[r + 1], dq1);
       }
       const float du = row16_sum(du0 + du1), dq = row16_sum(dq0 + dq1);
-      const float u = bb[tt] * (vv[tt][col] - du);
+      const float u = x.beta * (x.v - du);
 #pragma unroll
-      for (int r = 0; r < R; ++r) S[r] = fmaf(kk[tt][part * R + r], u, gg[tt][part * R + r] * S[r]);
-      if (part == 0) oo[tt][col] = fmaf(kqs[tt], u, dq);
+      for (int r = 0; r < R; ++r) S[r] = fmaf(x.kk[r], u, x.gg[r] * S[r]);
+      if (part == 0) oo[tt][col] = fmaf(x.kq, u, dq);
+    };
+    Operands xa, xb;
+    load(xa, 0);
+    for (int tt = 0; tt < n; tt += 2) {
+      if (tt + 1 < n) load(xb, tt + 1);
+      work(xa, tt);
+      if (tt + 1 < n) {
+        if (tt + 2 < n) load(xa, tt + 2);
+        work(xb, tt + 1);
+      }
     }
     block_sync_lds();
     if (vt < n && vj < Dv) a.out[(size_t)(tb + vt) * H * Dv + h * Dv + vj] = oo[vt][vc];

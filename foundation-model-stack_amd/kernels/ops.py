@@ -373,7 +373,8 @@ def attention(
             raise ValueError(f"score_slopes must be a contiguous float32 [{nheads}] tensor")
     if not (soft_cap >= 0.0 and math.isfinite(soft_cap)):
         raise ValueError(f"soft_cap {soft_cap} must be zero (none) or positive")
-    if q.dtype == torch.float32 or force_generic or head_dim % 16 or score_slopes is not None or value_dim:
+    if (q.dtype == torch.float32 or force_generic or head_dim % 16 or score_slopes is not None or value_dim
+            or (not decode and prefill_cap_is_generic(head_dim, soft_cap))):
         for t0 in range(0, T, 65535):
             n = min(65535, T - t0)
             check(lib.fmsamd_attn_generic(q[t0:].data_ptr(), q.stride(0), out[t0:].data_ptr(), out.stride(0), _code(q.dtype),
@@ -430,6 +431,12 @@ def decode_split(rows: int, n_pages: int):
     pages = -(-n_pages // splits)
     waves = max(1, min(8 if rows * splits <= 512 else 4, pages))
     return pages, waves
+
+
+def prefill_cap_is_generic(head_dim: int, soft_cap: float) -> bool:
+    """True if capped scores of this head size run the generic kernel in multi-token steps: the matrix-core prefill
+    kernel for head sizes between 64 and 128 has no cap."""
+    return soft_cap > 0.0 and 64 < head_dim < 128
 
 
 def prefill_qblock(nheads: int, kvheads: int, head_dim: int, n_tokens: int) -> int:

@@ -80,6 +80,8 @@ CONFIGS = {
     "D": dict(vocab=400, width=256, norm={"eps": 1e-6}, logit_scale=2.5, max_positions=2048, layers=[
         parallel(attention(4, 2, 128, 128, 100, 64, base=50000.0, softcap=25.0), delta(2, 1, 256, 32, 4), 1.0, 0.6, moe(4, 1, 64)),
         parallel(attention(8, 8, 32, 32, 64, 32, softcap=10.0), delta(8, 8, 32, 32, 4), 0.5, 1.0, None),
+        # a head size between 64 and 128: capped scores of prompts run the generic kernel, single tokens the matrix-core one
+        parallel(attention(2, 2, 96, 96, 50, 32, softcap=12.0), delta(1, 1, 16, 16, 3), 1.0, 1.0, moe(4, 2, 32)),
     ]),
 }
 
