@@ -83,6 +83,11 @@ CONFIGS = {
         # a head size between 64 and 128: capped scores of prompts run the generic kernel, single tokens the matrix-core one
         parallel(attention(2, 2, 96, 96, 50, 32, softcap=12.0), delta(1, 1, 16, 16, 3), 1.0, 1.0, moe(4, 2, 32)),
     ]),
+    # no attention at all: the cache has no pages to keep, only state
+    "E": dict(vocab=200, width=64, norm={"eps": 1e-6}, logit_scale=1.0, max_positions=512, layers=[
+        channel(delta(2, 2, 32, 16, 4, ranks=(8, 4)), moe(4, 2, 32)),
+        channel(delta(4, 1, 16, 8, 2, ranks=(4, 8)), None),
+    ]),
 }
 
 
