@@ -108,7 +108,7 @@ def write_folder(lib, folder, cfg_kw, seed, sharp=1.0):
     The experts' weights are not renormalized, so a router's choice that rounding turns moves a token's stream by much,
     and through the mixers every later token's: no comparison in bfloat16 would survive it.  The routers of these
     folders therefore decide by the token alone, and clearly: the stream's first channels (one per expert) hold, for
-    every token, a permutation of evenly spaced numbers; no branch writes into those channels; expert e's router row
+    every token, a permutation of numbers half a unit apart; no branch writes into those channels; expert e's router row
     reads channel e only.  (The router against arbitrary logits is tested by itself.)"""
     from fms_amd.weights import write_safetensors
 
@@ -136,7 +136,7 @@ def write_folder(lib, folder, cfg_kw, seed, sharp=1.0):
         elif k.endswith((".mix.b", ".right.b", ".left.g")):
             tensors[k] = t * 4  # gates and betas away from one half
     n_route = max([layer["mlp"]["router"]["experts"] for layer in cfg["layers"] if layer.get("mlp")] + [0])
-    levels = torch.linspace(-1.5, 1.5, max(n_route, 2))[:n_route]
+    levels = (torch.arange(n_route) - (n_route - 1) / 2) * 0.5  # half a unit apart, whatever the number of experts
     tensors["embed"][:, :n_route] = torch.stack([levels[torch.randperm(n_route, generator=gen)] for _ in range(cfg["vocab"])])
     for k in list(tensors):
         if k.endswith((".mix.o", ".left.o", ".right.o", ".down")):
