@@ -8,7 +8,7 @@
 #include "fmsamd.h"
 
 template <typename T, typename W>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
     qk_projection_norm_kernel(const float* __restrict__ proj, long ld, int nq, int nk, int nv, const W* __restrict__ wq,
                               const W* __restrict__ wk, float eps, T* __restrict__ out, long ldo,
                               const int* __restrict__ seq_of_token) {
@@ -35,7 +35,7 @@ extern "C" int fmsamd_qk_projection_norm(const float* proj, long ld, int nq, int
   FMS_REQUIRE(n_tokens > 0 && nq > 0 && nk > 0 && nv >= 0 && ld >= (long)nq + nk + nv && ldo >= (long)nq + nk + nv,
               "qk_projection_norm: bad sizes q=%d k=%d v=%d", nq, nk, nv);
 #define FMS_QKN(T, W)                                                                                                        \
-  qk_projection_norm_kernel<T, W><<<n_tokens, 256, 0, stream>>>(proj, ld, nq, nk, nv, (const W*)wq, (const W*)wk, eps, (T*)out, \
+  qk_projection_norm_kernel<T, W><<<n_tokens, n_tokens <= 64 ? 1024 : 256, 0, stream>>>(proj, ld, nq, nk, nv, (const W*)wq, (const W*)wk, eps, (T*)out, \
                                                                 ldo, seq_of_token)
   if (out_dtype == FMS_F32 && weight_dtype == FMS_F32) FMS_QKN(float, float);
   else if (out_dtype == FMS_BF16 && weight_dtype == FMS_F32) FMS_QKN(bf16, float);
@@ -48,7 +48,7 @@ extern "C" int fmsamd_qk_projection_norm(const float* proj, long ld, int nq, int
 }
 
 template <typename T>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
     gate_mul_kernel(const T* __restrict__ x, long ldx, const float* __restrict__ gate, long ldg, int act, float scale,
                     T* __restrict__ out, long ldo, int cols) {
   const int t = blockIdx.x;
@@ -64,10 +64,11 @@ extern "C" int fmsamd_gate_mul(const void* x, long ldx, const float* gate, long 
   if (n_tokens == 0) return 0;
   FMS_REQUIRE(n_tokens > 0 && cols > 0 && ldx >= cols && ldo >= cols && (gate == nullptr || ldg >= cols), "gate_mul: bad sizes");
   FMS_REQUIRE(act >= 0 && act <= FMS_ACT_LAST, "gate_mul: unknown activation %d", act);
+  const int threads = n_tokens <= 64 ? 1024 : 256;  // few tokens: fewer passes a thread, fewer round trips in a row
   if (dtype == FMS_F32)
-    gate_mul_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)x, ldx, gate, ldg, act, scale, (float*)out, ldo, cols);
+    gate_mul_kernel<float><<<n_tokens, threads, 0, stream>>>((const float*)x, ldx, gate, ldg, act, scale, (float*)out, ldo, cols);
   else if (dtype == FMS_BF16)
-    gate_mul_kernel<bf16><<<n_tokens, 256, 0, stream>>>((const bf16*)x, ldx, gate, ldg, act, scale, (bf16*)out, ldo, cols);
+    gate_mul_kernel<bf16><<<n_tokens, threads, 0, stream>>>((const bf16*)x, ldx, gate, ldg, act, scale, (bf16*)out, ldo, cols);
   else
     FMS_REQUIRE(false, "gate_mul: unknown dtype %d", dtype);
   FMS_LAUNCH_CHECK("gate_mul");

@@ -28,8 +28,23 @@
 __device__ __forceinline__ float softplus_f32(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 __device__ __forceinline__ float sigmoid_f32(float z) { return 1.f / (1.f + expf(-z)); }
 
+// How many tokens of its sequence come before token t in the step, up to taps - 1 (all that a convolution of `taps`
+// taps needs to know).  The candidates are loaded together, not one after another.
+__device__ __forceinline__ int tokens_before(const int* __restrict__ seq_of_token, int t, int seq, int taps) {
+  int prev[DELTA_MAX_TAPS - 1];
+#pragma unroll
+  for (int d = 1; d < DELTA_MAX_TAPS; ++d) prev[d - 1] = (d < taps && t - d >= 0) ? seq_of_token[t - d] : -2;
+  int have = 0;
+#pragma unroll
+  for (int d = 1; d < DELTA_MAX_TAPS; ++d)
+    if (have == d - 1 && prev[d - 1] == seq) have = d;
+  return have;
+}
+
+// Blocks of 1024 threads for steps of few tokens (a decode step has a block per token and nothing else to hide a
+// load's latency behind: the fewer passes a thread makes, the fewer round trips to memory follow one another).
 template <typename W>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
     delta_prepare_kernel(const float* __restrict__ proj, long ld, int col_b, const float* __restrict__ a, long lda, int col_a,
                          const W* __restrict__ conv_w, int taps, const float* __restrict__ a_log,
                          const float* __restrict__ dt_bias, const float* __restrict__ conv_state,
@@ -42,12 +57,7 @@ __global__ void __launch_bounds__(256)
   if (seq < 0) return;
   const int slot = slot_ids[seq];
   const int C = 2 * G * D + H * Dv;
-  // how many tokens of this sequence come before this one in the step (all that matters: up to taps - 1)
-  int have = 0;
-  for (int d = 1; d < taps; ++d) {
-    if (t - d >= 0 && seq_of_token[t - d] == seq) have = d;
-    else break;
-  }
+  const int have = tokens_before(seq_of_token, t, seq, taps);
   const float* state = conv_state + (size_t)slot * (taps - 1) * C;
   // two channels a thread and pass, all their taps asked for before any is used: a decode step has a block per token
   // and nothing else to hide a load's latency behind
@@ -103,18 +113,14 @@ __global__ void __launch_bounds__(256)
 
 // Runs after delta_prepare of the same step (which reads the old state).  The block of a sequence's last token of the
 // step writes; new entry s is either a row of the step or an old entry above s.
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
     conv_state_kernel(const float* __restrict__ proj, long ld, int taps, float* __restrict__ conv_state,
                       const int* __restrict__ seq_of_token, const int* __restrict__ slot_ids, int n_tokens, int C) {
   const int t = blockIdx.x;
   const int seq = seq_of_token[t];
   if (seq < 0) return;
   if (t + 1 < n_tokens && seq_of_token[t + 1] == seq) return;  // not the sequence's last token of the step
-  int have = 0;
-  for (int d = 1; d < taps; ++d) {
-    if (t - d >= 0 && seq_of_token[t - d] == seq) have = d;
-    else break;
-  }
+  const int have = tokens_before(seq_of_token, t, seq, taps);
   float* state = conv_state + (size_t)slot_ids[seq] * (taps - 1) * C;
   for (int c = threadIdx.x; c < C; c += blockDim.x) {
     float fresh[DELTA_MAX_TAPS - 1];  // all of a channel's new entries are read before any is written
@@ -328,8 +334,9 @@ extern "C" int fmsamd_delta_prepare(const float* proj, long ld, int col_b, const
   FMS_REQUIRE(C * 4 <= 64 * 1024, "delta_prepare: %ld channels do not fit one block's LDS", C);
   FMS_REQUIRE(col_a >= 0 && col_a + heads * (per_channel ? dim : 1) <= lda, "delta_prepare: the decay's columns leave its rows");
   const size_t lds = (size_t)C * sizeof(float);
+  const int threads = n_tokens <= 64 ? 1024 : 256;
 #define FMS_PREP(W)                                                                                                   \
-  delta_prepare_kernel<W><<<n_tokens, 256, lds, stream>>>(proj, ld, col_b, a, lda, col_a, (const W*)conv_w, taps, a_log, \
+  delta_prepare_kernel<W><<<n_tokens, threads, lds, stream>>>(proj, ld, col_b, a, lda, col_a, (const W*)conv_w, taps, a_log, \
                                                           dt_bias, conv_state, seq_of_token, slot_ids, qkv, beta, decay, \
                                                           kq, heads, kv_heads, dim, vdim, per_channel, q_scale)
   if (conv_dtype == FMS_F32) FMS_PREP(float);
@@ -338,7 +345,7 @@ extern "C" int fmsamd_delta_prepare(const float* proj, long ld, int col_b, const
 #undef FMS_PREP
   FMS_LAUNCH_CHECK("delta_prepare");
   if (taps > 1) {
-    conv_state_kernel<<<n_tokens, 256, 0, stream>>>(proj, ld, taps, conv_state, seq_of_token, slot_ids, n_tokens, (int)C);
+    conv_state_kernel<<<n_tokens, threads, 0, stream>>>(proj, ld, taps, conv_state, seq_of_token, slot_ids, n_tokens, (int)C);
     FMS_LAUNCH_CHECK("conv_state");
   }
   return 0;
@@ -346,7 +353,7 @@ extern "C" int fmsamd_delta_prepare(const float* proj, long ld, int col_b, const
 
 extern "C" int fmsamd_delta_rule(const float* qkv, const float* beta, const float* decay, const float* kq, float* state,
                                  float* out, const int* seq_starts, const int* seq_of_token, const int* slot_ids, int n_seqs, int heads,
-                                 int kv_heads, int dim, int vdim, int per_channel, hipStream_t stream) {
+                                 int kv_heads, int dim, int vdim, int per_channel, int single_tokens, hipStream_t stream) {
   if (n_seqs == 0) return 0;
   FMS_REQUIRE(n_seqs > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0,
               "delta_rule: bad sizes heads=%d kv_heads=%d dim=%d vdim=%d", heads, kv_heads, dim, vdim);
@@ -359,7 +366,14 @@ extern "C" int fmsamd_delta_rule(const float* qkv, const float* beta, const floa
     if (per_channel) delta_rule_kernel<R, TC, true><<<grid, DELTA_THREADS, 0, stream>>>(a);   \
     else delta_rule_kernel<R, TC, false><<<grid, DELTA_THREADS, 0, stream>>>(a);  \
   } while (0)
-  if (dim <= 2 * DELTA_PARTS) FMS_DR(2, 16);
+  // single_tokens: every sequence brings one token (a decode step).  Staging room for one pass of the block's threads
+  // is then enough, and a block that small leaves the compute unit's LDS to many more blocks.
+  if (single_tokens) {
+    if (dim <= 2 * DELTA_PARTS) FMS_DR(2, 8);
+    else if (dim <= 4 * DELTA_PARTS) FMS_DR(4, 4);
+    else if (dim <= 8 * DELTA_PARTS) FMS_DR(8, 2);
+    else FMS_DR(16, 1);
+  } else if (dim <= 2 * DELTA_PARTS) FMS_DR(2, 16);
   else if (dim <= 4 * DELTA_PARTS) FMS_DR(4, 16);
   else if (dim <= 8 * DELTA_PARTS) FMS_DR(8, 16);
   else FMS_DR(16, 8);

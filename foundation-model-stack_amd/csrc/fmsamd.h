@@ -265,10 +265,11 @@ int fmsamd_delta_prepare(const float* proj, long ld, int col_b, const float* a, 
                          int n_tokens, int heads, int kv_heads, int dim, int vdim, int per_channel, float q_scale,
                          hipStream_t stream);
 // The recurrence over every sequence's tokens of the step (seq_starts [n_seqs + 1]); state [slots][heads][vdim][dim]
-// is read and written; out [T, heads*vdim].
+// is read and written; out [T, heads*vdim].  single_tokens != 0: the caller knows that no sequence brings more than one
+// token, and the kernel stages accordingly (the result is the same either way).
 int fmsamd_delta_rule(const float* qkv, const float* beta, const float* decay, const float* kq, float* state, float* out,
                       const int* seq_starts, const int* seq_of_token, const int* slot_ids, int n_seqs, int heads,
-                      int kv_heads, int dim, int vdim, int per_channel, hipStream_t stream);
+                      int kv_heads, int dim, int vdim, int per_channel, int single_tokens, hipStream_t stream);
 // out[t, h, :] = o[t, h, :] / rms * weight * act(gate[t, h, :]) * out_scale
 int fmsamd_gated_head_norm(const float* o, const float* gate, long ldg, const void* weight, int weight_dtype, float eps,
                            int act, float out_scale, void* out, int out_dtype, long ldo, const int* seq_of_token,

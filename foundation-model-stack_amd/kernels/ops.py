@@ -1021,10 +1021,11 @@ def delta_prepare(proj: torch.Tensor, col_b: int, a: torch.Tensor, col_a: int, c
 
 def delta_rule(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, kq: torch.Tensor, state: torch.Tensor, seq_starts: torch.Tensor,
                seq_of_token: torch.Tensor, slot_ids: torch.Tensor, n_seqs: int, heads: int, kv_heads: int, dim: int, vdim: int,
-               per_channel: bool) -> torch.Tensor:
+               per_channel: bool, single_tokens: bool = False) -> torch.Tensor:
     """The recurrence S = g S; u = beta (v - S^T k); S += k u^T; o = S^T q over the tokens of every sequence of the
     step (kq [T, kv_heads] holds k . q of every token, as delta_prepare leaves it), from and into state [slots, heads, vdim, dim] (float32, S transposed) -> o float32 [T, heads*vdim].
-    Sequence b of the step owns the token rows seq_starts[b] .. seq_starts[b + 1] and the state of slot_ids[b]."""
+    Sequence b of the step owns the token rows seq_starts[b] .. seq_starts[b + 1] and the state of slot_ids[b].
+    single_tokens: every sequence brings one token (a decode step); the kernel then stages for that."""
     _need_cuda(qkv, beta, decay, kq, state, seq_starts, seq_of_token, slot_ids)
     for name, t in (("seq_starts", seq_starts), ("seq_of_token", seq_of_token), ("slot_ids", slot_ids)):
         _need_i32(name, t)
@@ -1043,7 +1044,7 @@ def delta_rule(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, kq: t
     out = torch.empty(T, heads * vdim, dtype=torch.float32, device=qkv.device)
     check(load().fmsamd_delta_rule(qkv.data_ptr(), beta.data_ptr(), decay.data_ptr(), kq.data_ptr(), state.data_ptr(), out.data_ptr(),
                                    seq_starts.data_ptr(), seq_of_token.data_ptr(), slot_ids.data_ptr(), n_seqs, heads, kv_heads, dim,
-                                   vdim, int(bool(per_channel)), _stream()))
+                                   vdim, int(bool(per_channel)), int(bool(single_tokens)), _stream()))
     return out
 
 

@@ -115,7 +115,7 @@ class GatedDeltaRule(Mixer):
         qkv, beta, decay, kq = ops.delta_prepare(proj, self.col_b, a, col_a, self.w["conv.weight"], self._a_log, self._dt_bias,
                                              state["conv"], batch.seq_of_token, batch.slot_ids, H, G, D, V, self.per_channel, D ** -0.5)
         o = ops.delta_rule(qkv, beta, decay, kq, state["S"], batch.seq_starts, batch.seq_of_token, batch.slot_ids, batch.n_seqs, H, G, D, V,
-                           self.per_channel)
+                           self.per_channel, single_tokens=batch.is_decode)
         normed = ops.gated_head_norm(o, gate, self.w["norm.weight"], self.eps, self.gate_activation, H, V, x.dtype, batch.seq_of_token,
                                      scale=out_scale, out=out)
         return BranchOutput(normed, self.out)

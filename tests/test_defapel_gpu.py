@@ -275,7 +275,7 @@ def test_delta_rule_whole_in_portions_and_in_a_batch(lib, sizes):
     S = torch.randn(n_slots, H, V, D, device=DEV)  # slots hold what earlier sequences left
     conv_state = torch.randn(n_slots, max(taps - 1, 1), C, device=DEV)
 
-    def run(pieces, slots):
+    def run(pieces, slots, single_tokens=False):
         """pieces: per sequence (proj rows, a rows); one step for all of them."""
         lens = [p.shape[0] for p, _ in pieces]
         seq = torch.repeat_interleave(torch.arange(len(pieces)), torch.tensor(lens)).to(torch.int32).to(DEV)
@@ -285,7 +285,7 @@ def test_delta_rule_whole_in_portions_and_in_a_batch(lib, sizes):
         aa = torch.cat([x for _, x in pieces]).to(DEV)
         qkv, beta, decay, kq = ops.delta_prepare(pr, C, aa, 1, conv_w.to(DEV), a_log.to(DEV), dt_bias.to(DEV), conv_state, seq, slot_ids,
                                                  H, G, D, V, per_channel, D ** -0.5)
-        out = ops.delta_rule(qkv, beta, decay, kq, S, starts, seq, slot_ids, len(pieces), H, G, D, V, per_channel)
+        out = ops.delta_rule(qkv, beta, decay, kq, S, starts, seq, slot_ids, len(pieces), H, G, D, V, per_channel, single_tokens=single_tokens)
         return torch.split(out.cpu(), lens)
 
     tol = dict(atol=5e-5, rtol=1e-4)
@@ -297,6 +297,11 @@ def test_delta_rule_whole_in_portions_and_in_a_batch(lib, sizes):
             got.append(run([(proj[at : at + n], a[at : at + n])], [2])[0])
             at += n
         torch.testing.assert_close(torch.cat(got), want, **tol)
+    # token by token as a decode step runs it (the kernel is told that no sequence brings more than one token)
+    S[2].zero_()
+    conv_state[2].zero_()
+    got = [run([(proj[t : t + 1], a[t : t + 1])], [2], single_tokens=True)[0] for t in range(40)]
+    torch.testing.assert_close(torch.cat(got), want[:40], **tol)
     # a batch of three unequal sequences in slots 3, 0, 1 (freshly zeroed, as the cache hands them out), then each goes on
     for s in (3, 0, 1):
         S[s].zero_()
