@@ -371,10 +371,10 @@ def design_comparison(args, design) -> int:
     watched = ["linear", "gated_linear", "linear_into_stream", "headwise_linear", "attention", "latent_attention", "moe_experts",
                "moe_route", "moe_combine", "add_norm", "norm_add_norm", "rms_norm_cols", "rope_kv_write", "qkv_rope_write",
                "latent_kv_write", "latent_q_rotate", "activation", "clamped_gated_act", "gated_act", "embed",
-               "delta_rule", "delta_prepare", "gated_head_norm", "qk_projection_norm", "gate_mul", "scale_", "cast"]
+               "delta_rule", "delta_prepare", "gated_head_norm", "qk_projection_norm", "gate_mul", "scale_", "cast", "cast_cols"]
     small = {"moe_route", "moe_combine", "add_norm", "norm_add_norm", "rms_norm_cols", "rope_kv_write", "latent_kv_write",
              "latent_q_rotate", "activation", "clamped_gated_act", "gated_act", "embed", "delta_prepare", "gated_head_norm",
-             "qk_projection_norm", "gate_mul", "scale_", "cast"}
+             "qk_projection_norm", "gate_mul", "scale_", "cast", "cast_cols"}
 
     def classes_of_a_step(run):
         """{class: (ms, ms at the roofline)} of the kernels of `run()`, by events around every call into the library."""

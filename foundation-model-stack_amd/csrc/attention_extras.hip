@@ -3,6 +3,7 @@
 //                       at once, before they are cut into heads and rotated), from the float32 sums of the projection;
 //                       the values are copied.  One rounding to the activation type.
 //   gate_mul:           out = x * act(gate) * scale (gate: float32 logits, or none), into rows of any stride.
+//   cast_cols:          a run of columns of float32 rows as rows of their own, in the activation type.
 //   scale_f32:          x *= s in place.
 #include "common.h"
 #include "fmsamd.h"
@@ -72,6 +73,24 @@ extern "C" int fmsamd_gate_mul(const void* x, long ldx, const float* gate, long 
   else
     FMS_REQUIRE(false, "gate_mul: unknown dtype %d", dtype);
   FMS_LAUNCH_CHECK("gate_mul");
+  return 0;
+}
+
+// out[t, 0:n] = x[t, col0 : col0 + n] in another type
+template <typename T>
+__global__ void __launch_bounds__(1024) cast_cols_kernel(const float* __restrict__ x, long ldx, T* __restrict__ out, long ldo, int n) {
+  const int t = blockIdx.x;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) out[(size_t)t * ldo + i] = from_f32<T>(x[(size_t)t * ldx + i]);
+}
+
+extern "C" int fmsamd_cast_cols(const float* x, long ldx, void* out, int out_dtype, long ldo, int n_tokens, int n, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  FMS_REQUIRE(n_tokens > 0 && n > 0 && ldx >= n && ldo >= n, "cast_cols: bad sizes");
+  const int threads = n >= 1024 ? 1024 : (n >= 256 ? 256 : 64);
+  if (out_dtype == FMS_F32) cast_cols_kernel<float><<<n_tokens, threads, 0, stream>>>(x, ldx, (float*)out, ldo, n);
+  else if (out_dtype == FMS_BF16) cast_cols_kernel<bf16><<<n_tokens, threads, 0, stream>>>(x, ldx, (bf16*)out, ldo, n);
+  else FMS_REQUIRE(false, "cast_cols: unknown dtype %d", out_dtype);
+  FMS_LAUNCH_CHECK("cast_cols");
   return 0;
 }
 

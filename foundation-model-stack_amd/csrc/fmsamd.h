@@ -252,6 +252,8 @@ int fmsamd_qk_projection_norm(const float* proj, long ld, int nq, int nk, int nv
 int fmsamd_gate_mul(const void* x, long ldx, const float* gate, long ldg, int act, float scale, void* out, long ldo,
                     int dtype, int n_tokens, int cols, hipStream_t stream);
 int fmsamd_scale_f32(float* x, long n, float s, hipStream_t stream);
+// out[t, 0:n] = x[t, 0:n] (x: float32 rows ldx apart, already offset to the first column) in out_dtype
+int fmsamd_cast_cols(const float* x, long ldx, void* out, int out_dtype, long ldo, int n_tokens, int n, hipStream_t stream);
 
 // ---- the gated delta rule (delta_rule.hip) ------------------------------------------------------------------------------
 // proj: float32 rows whose first C = 2*kv_heads*dim + heads*vdim columns are the q, k and v channels before the

@@ -62,6 +62,7 @@ _SIGNATURES = {
     "fmsamd_qk_projection_norm": [P, L, I, I, I, P, P, I, F, P, I, L, P, I, P],
     "fmsamd_gate_mul": [P, L, P, L, I, F, P, L, I, I, I, P],
     "fmsamd_scale_f32": [P, L, F, P],
+    "fmsamd_cast_cols": [P, L, P, I, L, I, I, P],
     "fmsamd_delta_prepare": [P, L, I, P, L, I, P, I, I, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, P],
     "fmsamd_delta_rule": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
     "fmsamd_gated_head_norm": [P, P, L, P, I, F, I, F, P, I, L, P, I, I, I, P],

@@ -961,6 +961,18 @@ def gate_mul(x: torch.Tensor, gate: Optional[torch.Tensor], activation: str = "s
     return out
 
 
+def cast_cols(x: torch.Tensor, col0: int, n: int, dtype: torch.dtype) -> torch.Tensor:
+    """The columns col0 .. col0 + n of float32 rows as a contiguous [T, n] tensor of `dtype` (one kernel, no copy before it)."""
+    _need_cuda(x)
+    _rows2d("x", x)
+    if x.dtype != torch.float32 or col0 < 0 or n <= 0 or col0 + n > x.shape[1]:
+        raise ValueError(f"cast_cols takes float32 rows and a run of columns inside them, got {x.dtype} {tuple(x.shape)} [{col0}, {col0 + n})")
+    out = torch.empty(x.shape[0], n, dtype=dtype, device=x.device)
+    view = x[:, col0 : col0 + n]
+    check(load().fmsamd_cast_cols(view.data_ptr(), x.stride(0), out.data_ptr(), _code(dtype), out.stride(0), x.shape[0], n, _stream()))
+    return out
+
+
 def scale_(x: torch.Tensor, s: float) -> torch.Tensor:
     """x *= s in place (contiguous float32)."""
     _need_cuda(x)

@@ -154,7 +154,7 @@ class MultiHeadAttention(Mixer):
                 qkv = ops.qk_projection_norm(proj, self.n_q, self.n_k, self.n_v, self.w["q_norm.weight"], self.w["k_norm.weight"],
                                              self.norm_eps, x.dtype, batch.seq_of_token)
             else:
-                qkv = ops.cast(proj[:, : self.n_q + self.n_k + self.n_v].contiguous(), x.dtype)
+                qkv = ops.cast_cols(proj, 0, self.n_q + self.n_k + self.n_v, x.dtype)
             if self.output_gate:
                 gate = proj[:, self.n_q + self.n_k + self.n_v :]
             if tables is None and self.position_encoder is not None:

@@ -103,12 +103,12 @@ class GatedDeltaRule(Mixer):
         # decays, gates, unit vectors and the recurrence are formed from the float32 sums of this product
         proj = self.in_proj.forward(x, out_dtype=torch.float32)
         if self.decay_rank:
-            low = ops.cast(proj[:, self.col_a : self.col_a + self.decay_rank].contiguous(), x.dtype)
+            low = ops.cast_cols(proj, self.col_a, self.decay_rank, x.dtype)
             a, col_a = self.decay_up.forward(low, out_dtype=torch.float32), 0
         else:
             a, col_a = proj, self.col_a
         if self.gate_rank:
-            low = ops.cast(proj[:, self.col_g : self.col_g + self.gate_rank].contiguous(), x.dtype)
+            low = ops.cast_cols(proj, self.col_g, self.gate_rank, x.dtype)
             gate = self.gate_up.forward(low, out_dtype=torch.float32)
         else:
             gate = proj[:, self.col_g : self.col_g + H * V]

@@ -395,6 +395,7 @@ def test_norm_over_whole_projections_gate_and_scales(lib, dtype):
     torch.testing.assert_close(out[:, 16:].float().cpu(), x.float() * torch.sigmoid(gate[:, 3:47]) * 0.8, **tol)
     logits = torch.randn(5, 33, generator=gen)
     torch.testing.assert_close(ops.scale_(logits.to(DEV), 1.75).cpu(), logits * 1.75)
+    torch.testing.assert_close(ops.cast_cols(proj.to(DEV), 3, 29, dtype).float().cpu(), proj[:, 3:32].to(dtype).float())
     # a norm whose weight is stored around zero
     from fms_amd.parts import make_part
 
