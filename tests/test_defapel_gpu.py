@@ -763,6 +763,21 @@ def test_command_line_and_trace_replay(lib, folders, tmp_path):
         judge(read(0), Expected.stack([want["x"][0], want["x"][79], want["y"][37]]), dtype)
         judge(read(2), Expected.stack([want["x"][81], want["y"][39]]), dtype)
         judge(read(10), want["x"][89:90], dtype)
+    # many short requests at once, --max-tokens counting their tokens as they are (every request still takes a page and a slot)
+    short = {f"s{i}": tokens_for(cfg["vocab"], 4 + i % 5, 60 + i) for i in range(14)}
+    steps = [{"step": 0, "entries": [{"id": k, "tokens": v[:-2], "want": [len(v) - 3]} for k, v in short.items()], "end": []}]
+    for j in (2, 1):
+        steps.append({"step": len(steps), "entries": [{"id": k, "tokens": [v[-j]], "want": [0]} for k, v in short.items()],
+                      "end": list(short) if j == 1 else []})
+    out_dir = str(tmp_path / "out_short")
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folders[name], "--dtype", "float32",
+                           "--out", out_dir, "--max-tokens", str(sum(len(v) for v in short.values()))],
+                          input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    want = {k: expect(cfg, weights, v, "float32") for k, v in short.items()}
+    for step, back in ((0, 3), (1, 2), (2, 1)):
+        got = torch.from_numpy(np.fromfile(os.path.join(out_dir, f"{step}.f32"), dtype="<f4").reshape(-1, cfg["vocab"]).copy())
+        judge(got, Expected.stack([want[k][len(v) - back] for k, v in short.items()]), "float32")
 
 
 def test_the_inference_program_and_a_model_from_the_registry(lib, folders):
