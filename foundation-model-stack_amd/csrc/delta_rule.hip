@@ -139,10 +139,8 @@ __global__ void __launch_bounds__(1024)
 // --------------------------------------------------------------------------
 // the recurrence
 // --------------------------------------------------------------------------
-#define DELTA_PARTS 16                      // lanes that share a column of S
 #define DELTA_WAVES 4                       // waves of a block: they share the staged tokens
 #define DELTA_THREADS (DELTA_WAVES * WAVE)
-#define DELTA_COLS (DELTA_THREADS / DELTA_PARTS)  // columns of S a block owns
 
 struct DeltaArgs {
   const float* qkv;    // [T, C]: q [G*D] | k [G*D] | v [H*Dv]
@@ -169,19 +167,39 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
-// R: rows of S per lane (D <= 16 R).  TC: tokens staged at a time.  A block's four waves own 16 columns of one head and
-// share the staged tokens (staging costs instructions, and four waves split them).  The next run's q, k and g are
-// asked for from global memory before this run is worked on and wait in registers meanwhile.
-template <int R, int TC, bool PER_CHANNEL>
+// The sum over the PARTS lanes that share a column: a row of 16 lanes, or two rows (the second step swaps the odd rows
+// of one copy with the even rows of another, so that their sum is the pair's sum in both).
+template <int PARTS>
+__device__ __forceinline__ float row_sum(float v) {
+  v = row16_sum(v);
+  if constexpr (PARTS == 32) {
+    const unsigned u = __float_as_uint(v);
+    const auto rows = __builtin_amdgcn_permlane16_swap(u, u, false, false);  // rows [0, 0, 2, 2] and [1, 1, 3, 3]
+    v = __uint_as_float(rows[0]) + __uint_as_float(rows[1]);
+  }
+  return v;
+}
+
+// PARTS: lanes that share a column of S (16, or 32 where a step has few sequences and heads: twice the blocks, half the
+// work a token and lane).  R: rows of S per lane (D <= PARTS R).  TC: tokens staged at a time.  A block's four waves own
+// 256 / PARTS columns of one head and share the staged tokens (staging costs instructions, and four waves split them).
+// The next run's q, k and g are asked for from global memory before this run is worked on and wait in registers meanwhile.
+template <int PARTS, int R, int TC, bool PER_CHANNEL>
 __global__ void __launch_bounds__(DELTA_THREADS) delta_rule_kernel(DeltaArgs a) {
+  constexpr int DELTA_COLS = DELTA_THREADS / PARTS;  // columns of S the block owns
+  constexpr int DELTA_PARTS = PARTS;
   constexpr int DP = R * DELTA_PARTS;          // padded key size
   constexpr int NI = TC * DP / DELTA_THREADS;  // staged elements a thread
   static_assert(TC * DP % DELTA_THREADS == 0 && TC * DELTA_COLS <= DELTA_THREADS, "the staging loops assume this");
+  // With a decay per channel: qg = g q, kg = g k, k and g.  With one decay per head the factor leaves the inner products
+  // (S^T (g k) = g S^T k): q and k alone are staged, and g as one number a token; half the LDS traffic.
+  constexpr int CH = PER_CHANNEL ? TC : 1;
   __shared__ __attribute__((aligned(16))) float qg[TC][DP];
-  __shared__ __attribute__((aligned(16))) float kg[TC][DP];
+  __shared__ __attribute__((aligned(16))) float kg[CH][DP];
   __shared__ __attribute__((aligned(16))) float kk[TC][DP];
-  __shared__ __attribute__((aligned(16))) float gg[TC][DP];
+  __shared__ __attribute__((aligned(16))) float gg[CH][DP];
   __shared__ float vv[TC][DELTA_COLS];
+  __shared__ float gs[TC];
   __shared__ float bb[TC];
   __shared__ float kqs[TC];
   __shared__ float oo[TC][DELTA_COLS];
@@ -204,7 +222,7 @@ __global__ void __launch_bounds__(DELTA_THREADS) delta_rule_kernel(DeltaArgs a) 
   for (int r = 0; r < R; ++r) S[r] = (live && part * R + r < D) ? srow[r] : 0.f;
 
   // what a lane fetches of a run: NI (q, k, g) triples, one value, and beta and k . q of one token
-  float pq[NI], pk[NI], pg[NI], pv = 0.f, pb = 0.f, pkq = 0.f;
+  float pq[NI], pk[NI], pg[PER_CHANNEL ? NI : 1], pv = 0.f, pb = 0.f, pkq = 0.f, pgs = 1.f;
   const int vt = lane / DELTA_COLS, vc = lane % DELTA_COLS;  // the (token, column) whose value and output this lane moves
   const int vj = blockIdx.z * DELTA_COLS + vc;
   auto fetch = [&](int tb) {
@@ -213,18 +231,23 @@ __global__ void __launch_bounds__(DELTA_THREADS) delta_rule_kernel(DeltaArgs a) 
       const int idx = it * DELTA_THREADS + lane;
       const int tt = idx / DP, i = idx % DP;
       const int t = tb + tt;
-      pq[it] = pk[it] = pg[it] = 0.f;
+      // past the run's last token (and past the key channels) a token that changes nothing: k = 0, g = 1
+      pq[it] = pk[it] = 0.f;
+      if constexpr (PER_CHANNEL) pg[it] = 1.f;
       if (t < t1 && i < D) {
         const float* row = a.qkv + (size_t)t * C;
         pq[it] = row[kh * D + i];
         pk[it] = row[G * D + kh * D + i];
-        pg[it] = PER_CHANNEL ? a.decay[((size_t)t * H + h) * D + i] : a.decay[(size_t)t * H + h];
+        if constexpr (PER_CHANNEL) pg[it] = a.decay[((size_t)t * H + h) * D + i];
       }
     }
+    pgs = 1.f;
+    pb = 0.f;
     pv = (vt < TC && tb + vt < t1 && vj < Dv) ? a.qkv[(size_t)(tb + vt) * C + 2 * G * D + h * Dv + vj] : 0.f;
     if (lane < TC && tb + lane < t1) {
       pb = a.beta[(size_t)(tb + lane) * H + h];
       pkq = a.kq[(size_t)(tb + lane) * G + kh];
+      if constexpr (!PER_CHANNEL) pgs = a.decay[(size_t)(tb + lane) * H + h];
     }
   };
   fetch(t0);
@@ -235,28 +258,35 @@ __global__ void __launch_bounds__(DELTA_THREADS) delta_rule_kernel(DeltaArgs a) 
     for (int it = 0; it < NI; ++it) {
       const int idx = it * DELTA_THREADS + lane;
       const int tt = idx / DP, i = idx % DP;
-      qg[tt][i] = pq[it] * pg[it];
-      kg[tt][i] = pk[it] * pg[it];
       kk[tt][i] = pk[it];
-      gg[tt][i] = pg[it];
+      if constexpr (PER_CHANNEL) {
+        qg[tt][i] = pq[it] * pg[it];
+        kg[tt][i] = pk[it] * pg[it];
+        gg[tt][i] = pg[it];
+      } else {
+        qg[tt][i] = pq[it];
+      }
     }
     if (vt < TC) vv[vt][vc] = pv;
-    if (lane < TC) bb[lane] = pb, kqs[lane] = pkq;
+    if (lane < TC) bb[lane] = pb, kqs[lane] = pkq, gs[lane] = pgs;
     block_sync_lds();
     if (tb + TC < t1) fetch(tb + TC);  // under way while this run is worked on
 
     // a token's operands are read from LDS into registers while the token before it is worked on (two sets, in turn)
     struct Operands {
-      float kg[R], qg[R], kk[R], gg[R], beta, v, kq;
+      float kg[PER_CHANNEL ? R : 1], qg[R], kk[R], gg[PER_CHANNEL ? R : 1], g, beta, v, kq;
     };
     auto load = [&](Operands& x, int tt) {
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        x.kg[r] = kg[tt][part * R + r];
         x.qg[r] = qg[tt][part * R + r];
         x.kk[r] = kk[tt][part * R + r];
-        x.gg[r] = gg[tt][part * R + r];
+        if constexpr (PER_CHANNEL) {
+          x.kg[r] = kg[tt][part * R + r];
+          x.gg[r] = gg[tt][part * R + r];
+        }
       }
+      x.g = gs[tt];
       x.beta = bb[tt];
       x.v = vv[tt][col];
       x.kq = kqs[tt];
@@ -265,24 +295,29 @@ __global__ void __launch_bounds__(DELTA_THREADS) delta_rule_kernel(DeltaArgs a) 
       float du0 = 0.f, du1 = 0.f, dq0 = 0.f, dq1 = 0.f;
 #pragma unroll
       for (int r = 0; r < R; r += 2) {
-        du0 = fmaf(S[r], x.kg[r], du0);
+        du0 = fmaf(S[r], PER_CHANNEL ? x.kg[PER_CHANNEL ? r : 0] : x.kk[r], du0);
         dq0 = fmaf(S[r], x.qg[r], dq0);
-        du1 = fmaf(S[r + 1], x.kg[r + 1], du1);
+        du1 = fmaf(S[r + 1], PER_CHANNEL ? x.kg[PER_CHANNEL ? r + 1 : 0] : x.kk[r + 1], du1);
         dq1 = fmaf(S[r + 1], x.qg[r + 1], dq1);
       }
-      const float du = row16_sum(du0 + du1), dq = row16_sum(dq0 + dq1);
+      float du = row_sum<PARTS>(du0 + du1), dq = row_sum<PARTS>(dq0 + dq1);
+      if constexpr (!PER_CHANNEL) du *= x.g, dq *= x.g;  // the head's decay, taken out of the sums
       const float u = x.beta * (x.v - du);
 #pragma unroll
-      for (int r = 0; r < R; ++r) S[r] = fmaf(x.kk[r], u, x.gg[r] * S[r]);
+      for (int r = 0; r < R; ++r) S[r] = fmaf(x.kk[r], u, (PER_CHANNEL ? x.gg[PER_CHANNEL ? r : 0] : x.g) * S[r]);
       if (part == 0) oo[tt][col] = fmaf(x.kq, u, dq);
     };
+    // Tokens go in pairs, and a run of an odd number works on one staged token that changes nothing (beta = 0, k = 0,
+    // g = 1; its output is not copied out): the loop's body then has no branch around its loads, and the compiler can
+    // let a token's work wait for its own operands only, not for the ones just asked for.
     Operands xa, xb;
     load(xa, 0);
-    for (int tt = 0; tt < n; tt += 2) {
-      if (tt + 1 < n) load(xb, tt + 1);
+    const int n2 = TC > 1 ? (n + 1) & ~1 : 1;
+    for (int tt = 0; tt < n2; tt += 2) {
+      load(xb, tt + 1 < TC ? tt + 1 : tt);
       work(xa, tt);
-      if (tt + 1 < n) {
-        if (tt + 2 < n) load(xa, tt + 2);
+      if constexpr (TC > 1) {
+        load(xa, tt + 2 < TC ? tt + 2 : tt);
         work(xb, tt + 1);
       }
     }
@@ -357,26 +392,34 @@ extern "C" int fmsamd_delta_rule(const float* qkv, const float* beta, const floa
   if (n_seqs == 0) return 0;
   FMS_REQUIRE(n_seqs > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0,
               "delta_rule: bad sizes heads=%d kv_heads=%d dim=%d vdim=%d", heads, kv_heads, dim, vdim);
-  FMS_REQUIRE(dim <= 16 * DELTA_PARTS, "delta_rule: %d key channels (at most %d)", dim, 16 * DELTA_PARTS);
-  FMS_REQUIRE(heads <= 65535 && ceil_div(vdim, DELTA_COLS) <= 65535, "delta_rule: too many heads or value channels for one launch");
+  FMS_REQUIRE(dim <= 256, "delta_rule: %d key channels (at most 256)", dim);
   DeltaArgs a{qkv, beta, decay, kq, state, out, seq_starts, seq_of_token, slot_ids, heads, kv_heads, dim, vdim, per_channel};
-  const dim3 grid(n_seqs, heads, ceil_div(vdim, DELTA_COLS));
-#define FMS_DR(R, TC)                                                                       \
-  do {                                                                                      \
-    if (per_channel) delta_rule_kernel<R, TC, true><<<grid, DELTA_THREADS, 0, stream>>>(a);   \
-    else delta_rule_kernel<R, TC, false><<<grid, DELTA_THREADS, 0, stream>>>(a);  \
+  // Few sequences and heads (a prompt alone): 32 lanes a column instead of 16, so that the step has twice the blocks and a
+  // token costs every wave half the work; with many blocks anyway, 16 lanes (fewer reduction steps a token).
+  const bool wide = !single_tokens && dim > 32 && (long)n_seqs * heads * ceil_div(vdim, 16) <= 512;
+  const int cols = DELTA_THREADS / (wide ? 32 : 16);
+  FMS_REQUIRE(heads <= 65535 && ceil_div(vdim, cols) <= 65535, "delta_rule: too many heads or value channels for one launch");
+  const dim3 grid(n_seqs, heads, ceil_div(vdim, cols));
+#define FMS_DR(P, R, TC)                                                                        \
+  do {                                                                                          \
+    if (per_channel) delta_rule_kernel<P, R, TC, true><<<grid, DELTA_THREADS, 0, stream>>>(a);  \
+    else delta_rule_kernel<P, R, TC, false><<<grid, DELTA_THREADS, 0, stream>>>(a);             \
   } while (0)
   // single_tokens: every sequence brings one token (a decode step).  Staging room for one pass of the block's threads
   // is then enough, and a block that small leaves the compute unit's LDS to many more blocks.
   if (single_tokens) {
-    if (dim <= 2 * DELTA_PARTS) FMS_DR(2, 8);
-    else if (dim <= 4 * DELTA_PARTS) FMS_DR(4, 4);
-    else if (dim <= 8 * DELTA_PARTS) FMS_DR(8, 2);
-    else FMS_DR(16, 1);
-  } else if (dim <= 2 * DELTA_PARTS) FMS_DR(2, 16);
-  else if (dim <= 4 * DELTA_PARTS) FMS_DR(4, 16);
-  else if (dim <= 8 * DELTA_PARTS) FMS_DR(8, 16);
-  else FMS_DR(16, 8);
+    if (dim <= 32) FMS_DR(16, 2, 8);
+    else if (dim <= 64) FMS_DR(16, 4, 4);
+    else if (dim <= 128) FMS_DR(16, 8, 2);
+    else FMS_DR(16, 16, 1);
+  } else if (wide) {
+    if (dim <= 64) FMS_DR(32, 2, 16);
+    else if (dim <= 128) FMS_DR(32, 4, 16);
+    else FMS_DR(32, 8, 8);
+  } else if (dim <= 32) FMS_DR(16, 2, 16);
+  else if (dim <= 64) FMS_DR(16, 4, 16);
+  else if (dim <= 128) FMS_DR(16, 8, 16);
+  else FMS_DR(16, 16, 8);
 #undef FMS_DR
   FMS_LAUNCH_CHECK("delta_rule");
   return 0;

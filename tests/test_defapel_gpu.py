@@ -254,7 +254,9 @@ def _plain_delta(proj, a, conv_w, a_log, dt_bias, H, G, D, V, per_channel, C):
 
 
 @pytest.mark.parametrize("sizes", [(4, 2, 16, 24, 3, False), (2, 1, 40, 20, 4, True), (3, 3, 20, 12, 1, True), (2, 2, 128, 64, 4, False),
-                                   (1, 1, 160, 10, 2, True), (2, 1, 256, 33, 8, False), (5, 5, 32, 7, 4, True), (3, 1, 64, 130, 5, False)])
+                                   (1, 1, 160, 10, 2, True), (2, 1, 256, 33, 8, False), (5, 5, 32, 7, 4, True), (3, 1, 64, 130, 5, False),
+                                   # so many heads and value channels that a column gets 16 lanes instead of 32
+                                   (32, 32, 64, 272, 2, False), (36, 12, 40, 240, 3, True)])
 def test_delta_rule_whole_in_portions_and_in_a_batch(lib, sizes):
     """The convolution, the unit vectors, the gates and the recurrence of one sequence: whole, cut into portions down to
     one and two tokens (the state carries over), and beside two other sequences in slots used before."""
