@@ -11,12 +11,12 @@
 //                   beta = sigmoid, g = exp(-exp(A_log) softplus(a + dt_bias)).
 //   conv_state:     the last (taps - 1) inputs of every sequence go into its state.
 //   delta_rule:     the recurrence.  Columns of S never mix (each value channel is a recurrence of its own), so a wave
-//                   owns a few columns of one head of one sequence: 16 lanes share a column, each with a run of its
-//                   rows in registers.  The wave walks over the sequence's tokens; q, k and g of a run of tokens are
+//                   owns a few columns of one head of one sequence: 16 (or 32) lanes share a column, each with a run of
+//                   its rows in registers.  The wave walks over the sequence's tokens; q, k and g of a run of tokens are
 //                   staged in LDS for all its lanes (the next run's are asked for before this one is worked on).  With
 //                   kg = g k and qg = g q, both inner products of a token read the state as the token found it,
-//                   u = beta (v - S^T kg),  o = S^T qg + (k . q) u,  and are summed over the 16 lanes together, in the
-//                   vector unit; then S <- g S + k u^T.
+//                   u = beta (v - S^T kg),  o = S^T qg + (k . q) u,  and are summed over the column's lanes together, in
+//                   the vector unit; then S <- g S + k u^T.  (A decay per head leaves the sums: g S^T k.)
 //   gated_head_norm: o / rms(o) * weight * act(gate) per head, rounded once to the activation type.
 //
 // The state is kept transposed, [slot][head][value channel][key channel], so that a lane's rows are contiguous.
